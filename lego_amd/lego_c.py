@@ -1,0 +1,44 @@
+"""C expression printer for LEGO index expressions (reference: lego/lego_c.py:5-38).
+
+Integer semantics throughout: ``floor(a/b)`` is ``/`` on non-negative ints, ``x**2`` is
+``x*x``.  Unlike the reference, which inherits ``fmin``/``fmax`` from the C99 printer,
+``Min``/``Max`` are printed as integer ternaries, because index expressions are integers.
+"""
+from sympy.printing.c import C99CodePrinter
+from sympy.printing.precedence import precedence
+
+from .lego import *  # noqa: F401,F403
+
+
+class LEGOCCodePrinter(C99CodePrinter):
+    def __init__(self, settings=None, **kwargs):
+        merged = dict(settings or {})
+        merged.update(kwargs)
+        super().__init__(merged)
+
+    def _print_floor(self, expr):
+        num, den = expr.args[0].as_numer_denom()
+        return f"(({self._print(num)})/({self._print(den)}))"
+
+    def _print_Pow(self, expr):
+        if expr.exp.is_Integer and 2 <= int(expr.exp) <= 4:
+            base = self.parenthesize(expr.base, precedence(expr))
+            return "*".join([base] * int(expr.exp))
+        return super()._print_Pow(expr)
+
+    def _fold_minmax(self, args, op):
+        out = self._print(args[0])
+        for a in args[1:]:
+            b = self._print(a)
+            out = f"(({out}) {op} ({b}) ? ({out}) : ({b}))"
+        return out
+
+    def _print_Min(self, expr):
+        return self._fold_minmax(expr.args, "<")
+
+    def _print_Max(self, expr):
+        return self._fold_minmax(expr.args, ">")
+
+    def _print_BitXor(self, expr):
+        a, b = expr.args
+        return f"(({self._print(a)}) ^ ({self._print(b)}))"

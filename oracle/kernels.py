@@ -1,0 +1,81 @@
+"""TEST INFRASTRUCTURE -- CPU oracle for the five lego_hip kernels.  Not part of the product.
+
+The reference's CPU path is "index expressions printed by ``lego_python`` and evaluated
+over index vectors, plus PyTorch CPU operators".  Each function restates one kernel that
+way and names what it follows:
+
+``transpose``      benchmarks/mlir/transpose_smem.py:28-80 -- ``B[wby,wbx,i,j,..] = A[rby,rbx,j,i,..]``
+                   over all logical indices, i.e. a gather/scatter through two layouts;
+                   the reference's own check is ``gold[j*nx+i] = in[i*nx+j]``
+                   (mlir_generated/transpose/transpose.cu:199-206).
+``softmax``        triton_generated/softmax/softmax.py:33-58, checked there against
+                   ``torch.softmax(x, axis=1)`` (:237-241).
+``layernorm_fwd``  triton_generated/layernorm/layernorm.py:57-101 (mean, biased variance,
+                   ``rstd = 1/sqrt(var+eps)``, ``y = (x-mean)*rstd*w + b``), checked there
+                   against ``torch.nn.functional.layer_norm`` (:446).
+``gemm``           triton_generated/matmul/matmul_NTA_NTB.py:97-122, checked against
+                   ``torch.matmul`` (:252).
+``grouped_gemm``   triton_generated/grouped_gemm/grouped_gemm.py:38-116, per problem
+                   ``torch.matmul`` (:316-350).
+
+Floating point oracles accumulate in fp32 and round once to fp16, which is what the
+tolerances of the parity tests are stated against.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from . import lego_index as li
+
+
+def transpose_layouts(rows, cols, tile_r, tile_c):
+    """Source (row-major) and destination (column-major) tiled layouts of a
+    ``rows x cols`` matrix, logical index ``(tile_i, tile_j, i, j)``."""
+    levels = ([rows // tile_r, cols // tile_c], [tile_r, tile_c])
+    return (li.tile_by(li.Order(li.row(rows, cols)), *levels),
+            li.tile_by(li.Order(li.col(rows, cols)), *levels))
+
+
+def transpose(x: torch.Tensor, tile_r: int, tile_c: int) -> torch.Tensor:
+    """Move every element from its offset in the row-major layout to the offset of the
+    same logical index in the column-major layout.  The result, read as a row-major
+    ``cols x rows`` matrix, is the transpose."""
+    rows, cols = x.shape
+    src, dst = transpose_layouts(rows, cols, tile_r, tile_c)
+    out = torch.empty(rows * cols, dtype=x.dtype)
+    src_off = torch.from_numpy(np.array(src.offsets()).reshape(-1))
+    dst_off = torch.from_numpy(np.array(dst.offsets()).reshape(-1))
+    out[dst_off] = x.reshape(-1)[src_off]
+    return out.view(cols, rows)
+
+
+def softmax(x: torch.Tensor) -> torch.Tensor:
+    return torch.softmax(x.float(), dim=-1).to(x.dtype)
+
+
+def layernorm_fwd(x, weight, bias, eps=1e-5):
+    """Returns ``(y, mean, rstd)`` with fp32 statistics."""
+    xf = x.float()
+    mean = xf.mean(dim=-1)
+    var = xf.var(dim=-1, unbiased=False)
+    rstd = torch.rsqrt(var + eps)
+    y = torch.nn.functional.layer_norm(xf, (x.shape[-1],), weight.float(), bias.float(), eps)
+    return y.to(x.dtype), mean, rstd
+
+
+def gemm(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    return (a.float() @ b.float()).to(a.dtype)
+
+
+def grouped_gemm(group_a, group_b):
+    return [gemm(a, b) for a, b in zip(group_a, group_b)]
+
+
+def grouped_pid(pid, num_pid_m, num_pid_n, group_m):
+    """Textbook grouped launch order (triton_generated/matmul/matmul_NTA_NTB.py:176-181)."""
+    width = group_m * num_pid_n
+    group_id = pid // width
+    first_m = group_id * group_m
+    size_m = np.minimum(num_pid_m - first_m, group_m)
+    return first_m + (pid % width) % size_m, (pid % width) // size_m
