@@ -1,0 +1,69 @@
+/* lego_hip.h -- C ABI of liblego_hip.so, the MI355X (gfx950) kernels generated from LEGO
+ * layouts by lego_amd.  Plain pointers and sizes only.
+ *
+ * Conventions for every entry point
+ *   - returns 0 on success, otherwise a hipError_t value (1 = hipErrorInvalidValue for a
+ *     null pointer, a misaligned base, or a shape the generated kernels do not cover);
+ *   - all tensor pointers are BORROWED DEVICE pointers, 16-byte aligned, row-major and
+ *     contiguous; nothing is allocated, freed or synchronised: the kernel is enqueued on
+ *     `stream` (a hipStream_t; NULL = the default stream) and the call returns;
+ *   - stateless and re-entrant: safe from several host threads on distinct streams.
+ *
+ * The reference has no FFI: its kernels are reached through generated Python host
+ * functions.  Each entry point below names the reference host function it stands behind.
+ */
+#ifndef LEGO_HIP_H
+#define LEGO_HIP_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ABI version of this header. */
+int lego_hip_abi_version(void);
+
+/* out[c][r] = in[r][c] for a rows x cols matrix; out is cols x rows.
+ * Replaces the generated transpose programs (reference: benchmarks/mlir/transpose_smem.py:28-80,
+ * mlir_generated/transpose/transpose_smem_4096.mlir:24-97), which have no callable entry.
+ * rows and cols must be multiples of 64. */
+int lego_hip_transpose_f32(const void* in, void* out, int rows, int cols, void* stream);
+int lego_hip_transpose_f16(const void* in, void* out, int rows, int cols, void* stream);
+
+/* y = softmax(x) over the last dimension of an M x N fp16 matrix, fp32 arithmetic.
+ * Replaces softmax(x) (reference: triton_generated/softmax/softmax.py:97-160).
+ * N must be a multiple of 8 and at most 16384. */
+int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream);
+
+/* LayerNorm forward over the last dimension of an M x N fp16 matrix; w, b are fp16 [N];
+ * mean, rstd are fp32 [M] outputs.  Replaces LEGOLayerNorm.forward / lego_layer_norm
+ * (reference: triton_generated/layernorm/layernorm.py:279-307).
+ * N must be a multiple of 8 and at most 16384. */
+int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void* b,
+                               float* mean, float* rstd, int M, int N, float eps, void* stream);
+
+/* C = A * B, A is M x K, B is K x N, C is M x N, fp16 with fp32 accumulation.
+ * Replaces matmul(a, b) (reference: triton_generated/matmul/matmul_NTA_NTB.py:129-145).
+ * Like the reference kernel (no edge masks, matmul_sympy.py:196-203) the sizes must divide
+ * the tiles: M and N multiples of 256, K a multiple of 64. */
+int lego_hip_gemm_f16(const void* a, const void* b, void* c, int M, int N, int K, void* stream);
+
+/* groups independent GEMMs in one launch.  a, b, c are HOST arrays of `groups` device
+ * pointers; sizes3 is a HOST array of groups*3 ints (M, N, K per problem).  At most 64
+ * groups; every M, N a multiple of 256 and K a multiple of 64.  Replaces
+ * lego_group_gemm_fn(group_A, group_B) (reference:
+ * triton_generated/grouped_gemm/grouped_gemm.py:120-162), whose device-side tables are
+ * passed here by value as kernel arguments, so no table is allocated or copied. */
+int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* const* c,
+                              const int* sizes3, int groups, void* stream);
+
+/* Tuning entry points: as above, with the launch shape chosen by the caller
+ * (waves_per_row in {1, 2, 4}).  Used by the benchmark to compare variants. */
+int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per_row, void* stream);
+int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const void* b,
+                                   float* mean, float* rstd, int M, int N, float eps,
+                                   int waves_per_row, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LEGO_HIP_H */

@@ -1,0 +1,106 @@
+"""Generates the HIP sources from the LEGO layouts and builds liblego_hip.so for gfx950.
+
+    python -m lego_amd.build            # generate + compile
+    python -m lego_amd.build --emit     # generate only
+
+Generated text goes to lego_amd/csrc/generated/, the library to lego_amd/lib/.  hipcc
+cross-compiles without a GPU.
+"""
+from __future__ import annotations
+
+import argparse
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+from .kernels import gemm, rowwise, transpose
+from .kernels.common import BANNER, CSRC, GENERATED
+from .lego_hip import HIPCC_FLAGS, hipcc_path
+
+ROOT = Path(__file__).resolve().parents[1]
+LIB_DIR = Path(__file__).resolve().parent / "lib"
+LIB_PATH = LIB_DIR / "liblego_hip.so"
+OBJ_DIR = LIB_DIR / "obj"
+
+# the tilings the library is built with
+TRANSPOSE_F32 = dict(dtype="f32", tile=(32, 32), group=(2, 2))
+TRANSPOSE_F16 = dict(dtype="f16", tile=(64, 64), group=(1, 1))
+ROWWISE_WAVES = (1, 2, 4)
+ROWWISE_DEFAULT_WAVES = 4
+ROWWISE_MAX_N = 16384
+GEMM = dict(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8)
+
+
+def generate():
+    """Write every generated source; returns the list of .hip paths to compile."""
+    units = []
+    t32, m32 = transpose.emit(**TRANSPOSE_F32)
+    t16, m16 = transpose.emit(**TRANSPOSE_F16)
+    units += [t32, t16]
+    units += [rowwise.emit(w) for w in ROWWISE_WAVES]
+    g, mg = gemm.emit(**GEMM)
+    units.append(g)
+
+    h = [f"// {BANNER}", "#pragma once", "#include <hip/hip_runtime.h>", ""]
+    h += [f"hipError_t {m32['kernel']}_launch(const void*, void*, int, int, hipStream_t);",
+          f"hipError_t {m16['kernel']}_launch(const void*, void*, int, int, hipStream_t);",
+          f"#define LEGO_TRANSPOSE_F32_LAUNCH {m32['kernel']}_launch",
+          f"#define LEGO_TRANSPOSE_F32_SR {m32['SR']}", f"#define LEGO_TRANSPOSE_F32_SC {m32['SC']}",
+          f"#define LEGO_TRANSPOSE_F16_LAUNCH {m16['kernel']}_launch",
+          f"#define LEGO_TRANSPOSE_F16_SR {m16['SR']}", f"#define LEGO_TRANSPOSE_F16_SC {m16['SC']}", ""]
+    for w in ROWWISE_WAVES:
+        h += [f"hipError_t lego_softmax_f16_w{w}_launch(const void*, void*, int, int, hipStream_t);",
+              f"hipError_t lego_layernorm_fwd_f16_w{w}_launch(const void*, void*, const void*, const void*, "
+              "float*, float*, int, int, float, hipStream_t);"]
+    h += [f"#define LEGO_ROWWISE_MAX_N {ROWWISE_MAX_N}",
+          "// waves per row: one wave keeps short rows free of barriers, four waves keep the",
+          "// register footprint of long rows small enough for full occupancy",
+          f"inline int lego_rowwise_default_wpr(int n) {{ return n <= 2048 ? 1 : {ROWWISE_DEFAULT_WAVES}; }}", ""]
+    h += ["hipError_t lego_gemm_f16_launch(const void*, const void*, void*, int, int, int, hipStream_t);",
+          "hipError_t lego_grouped_gemm_f16_launch(const void* const*, const void* const*, void* const*, "
+          "const int*, int, hipStream_t);",
+          f"#define LEGO_GEMM_BM {mg['BM']}", f"#define LEGO_GEMM_BN {mg['BN']}", f"#define LEGO_GEMM_BK {mg['BK']}",
+          f"#define LEGO_GROUPED_MAX_GROUPS {mg['MAX_GROUPS']}", ""]
+    GENERATED.mkdir(parents=True, exist_ok=True)
+    header = GENERATED / "launchers.h"
+    text = "\n".join(h)
+    if not header.exists() or header.read_text() != text:
+        header.write_text(text)
+    return [u.write() for u in units]
+
+
+def _compile(src: Path) -> Path:
+    obj = OBJ_DIR / (src.stem + ".o")
+    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", str(ROOT / "include"), "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src.name}:\n{res.stderr}")
+    return obj
+
+
+def build(verbose=True):
+    """Generate, compile every translation unit for gfx950 and link liblego_hip.so."""
+    sources = generate() + [CSRC / "lego_hip_abi.hip"]
+    OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=8) as pool:
+        objs = list(pool.map(_compile, sources))
+    cmd = [hipcc_path(), f"--offload-arch=gfx950", "-shared", "-fPIC", *[str(o) for o in objs], "-o", str(LIB_PATH)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stderr}")
+    if verbose:
+        print(f"built {LIB_PATH} from {len(sources)} translation units")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--emit", action="store_true", help="generate sources only")
+    ns = ap.parse_args()
+    if ns.emit:
+        for p in generate():
+            print(p)
+    else:
+        build()
+    sys.exit(0)

@@ -1,0 +1,99 @@
+// C-ABI entry points of liblego_hip.so (declared in include/lego_hip.h).
+//
+// This file is written by hand; the kernels and their launchers are generated from LEGO
+// layouts (python -m lego_amd.build) into csrc/generated/ and declared in
+// generated/launchers.h.  An entry point validates what the generated code assumes --
+// non-null, 16-byte aligned pointers and shapes that divide the tiles -- and enqueues one
+// kernel on the caller's stream.  It allocates nothing and never synchronises.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "lego_hip.h"
+#include "generated/launchers.h"
+
+namespace {
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool usable(const void* p) { return p != nullptr && aligned16(p); }
+inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
+inline int ok_or(hipError_t e) { return static_cast<int>(e); }
+constexpr int kInvalid = static_cast<int>(hipErrorInvalidValue);
+
+}  // namespace
+
+extern "C" {
+
+int lego_hip_abi_version(void) { return 1; }
+
+int lego_hip_transpose_f32(const void* in, void* out, int rows, int cols, void* stream)
+{
+  if (!usable(in) || !usable(out) || in == out) return kInvalid;
+  if (rows <= 0 || cols <= 0 || rows % LEGO_TRANSPOSE_F32_SR || cols % LEGO_TRANSPOSE_F32_SC) return kInvalid;
+  return ok_or(LEGO_TRANSPOSE_F32_LAUNCH(in, out, rows, cols, as_stream(stream)));
+}
+
+int lego_hip_transpose_f16(const void* in, void* out, int rows, int cols, void* stream)
+{
+  if (!usable(in) || !usable(out) || in == out) return kInvalid;
+  if (rows <= 0 || cols <= 0 || rows % LEGO_TRANSPOSE_F16_SR || cols % LEGO_TRANSPOSE_F16_SC) return kInvalid;
+  return ok_or(LEGO_TRANSPOSE_F16_LAUNCH(in, out, rows, cols, as_stream(stream)));
+}
+
+int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per_row, void* stream)
+{
+  if (!usable(x) || !usable(y)) return kInvalid;
+  if (M <= 0 || N <= 0 || N % 8 || N > LEGO_ROWWISE_MAX_N) return kInvalid;
+  switch (waves_per_row) {
+    case 1: return ok_or(lego_softmax_f16_w1_launch(x, y, M, N, as_stream(stream)));
+    case 2: return ok_or(lego_softmax_f16_w2_launch(x, y, M, N, as_stream(stream)));
+    case 4: return ok_or(lego_softmax_f16_w4_launch(x, y, M, N, as_stream(stream)));
+    default: return kInvalid;
+  }
+}
+
+int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream)
+{
+  return lego_hip_softmax_f16_wpr(x, y, M, N, lego_rowwise_default_wpr(N), stream);
+}
+
+int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const void* b,
+                                   float* mean, float* rstd, int M, int N, float eps,
+                                   int waves_per_row, void* stream)
+{
+  if (!usable(x) || !usable(y) || !usable(w) || !usable(b) || mean == nullptr || rstd == nullptr) return kInvalid;
+  if (M <= 0 || N <= 0 || N % 8 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
+  switch (waves_per_row) {
+    case 1: return ok_or(lego_layernorm_fwd_f16_w1_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+    case 2: return ok_or(lego_layernorm_fwd_f16_w2_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+    case 4: return ok_or(lego_layernorm_fwd_f16_w4_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+    default: return kInvalid;
+  }
+}
+
+int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void* b,
+                               float* mean, float* rstd, int M, int N, float eps, void* stream)
+{
+  return lego_hip_layernorm_fwd_f16_wpr(x, y, w, b, mean, rstd, M, N, eps, lego_rowwise_default_wpr(N), stream);
+}
+
+int lego_hip_gemm_f16(const void* a, const void* b, void* c, int M, int N, int K, void* stream)
+{
+  if (!usable(a) || !usable(b) || !usable(c)) return kInvalid;
+  if (M <= 0 || N <= 0 || K <= 0 || M % LEGO_GEMM_BM || N % LEGO_GEMM_BN || K % LEGO_GEMM_BK) return kInvalid;
+  return ok_or(lego_gemm_f16_launch(a, b, c, M, N, K, as_stream(stream)));
+}
+
+int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* const* c,
+                              const int* sizes3, int groups, void* stream)
+{
+  if (a == nullptr || b == nullptr || c == nullptr || sizes3 == nullptr) return kInvalid;
+  if (groups <= 0 || groups > LEGO_GROUPED_MAX_GROUPS) return kInvalid;
+  for (int g = 0; g < groups; ++g) {
+    const int m = sizes3[3 * g], n = sizes3[3 * g + 1], k = sizes3[3 * g + 2];
+    if (!usable(a[g]) || !usable(b[g]) || !usable(c[g])) return kInvalid;
+    if (m <= 0 || n <= 0 || k <= 0 || m % LEGO_GEMM_BM || n % LEGO_GEMM_BN || k % LEGO_GEMM_BK) return kInvalid;
+  }
+  return ok_or(lego_grouped_gemm_f16_launch(a, b, c, sizes3, groups, as_stream(stream)));
+}
+
+}  // extern "C"

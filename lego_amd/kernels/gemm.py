@@ -1,0 +1,149 @@
+"""Generator of the fp16 GEMM and grouped GEMM kernels.
+
+What LEGO contributes is what it contributes to the reference's Triton kernels
+(benchmarks/triton/matmul_sympy.py:37-78, grouped_gemm_sympy.py:7-24): the offsets of the
+A, B and C tiles of ``OrderBy(Row(..)).TileBy([M/BM, K/BK], [BM, BK])`` and friends, and the
+grouped launch order ``OrderBy(Col(max(npm//GM,1),1), Col(min(npm,GM),npn)).TileBy([npm,npn]).inv(pid)``.
+Here the same algebra also lays out what Triton hides: the lane-to-chunk assignment of
+the global loads, the XOR-rotated LDS tiles (``GenP`` blocks), the MFMA operand
+fragments, the accumulator-to-C map and the remap of workgroup ids onto the eight XCDs.
+
+The grouped kernel runs one workgroup per tile of every problem; a workgroup finds its
+problem from running tile totals passed as kernel arguments (the reference's kernel
+scans the same totals on the device, triton_generated/grouped_gemm/grouped_gemm.py:61-82)
+and then applies the grouped launch order inside that problem.
+"""
+from __future__ import annotations
+
+import sympy as sp
+
+from ..lego import BitXor, Col, GenP, OrderBy, Row
+from .common import BANNER, Emitted, code, idx, size, template, tidy
+
+XCDS = 8
+MAX_GROUPS = 64
+
+
+def lds_a_layout(bm, chunks):
+    """A tile in 16-byte chunks: ``row*chunks + (chunk ^ ((row//2) % chunks))``.
+
+    Sixteen lanes that read the same chunk of sixteen consecutive rows (one quarter of a
+    ds_read_b128) land on sixteen different 16-byte slots of the 256-byte bank window,
+    and so do the sixteen lanes that write two whole rows."""
+    def key(row):
+        return (row // 2) % chunks
+
+    def forward(rc):
+        row, ch = rc
+        return row * chunks + BitXor(sp.sympify(ch), sp.sympify(key(row)))
+
+    def backward(flat):
+        row, p = flat // chunks, flat % chunks
+        return (row, BitXor(sp.sympify(p), sp.sympify(key(row))))
+
+    return OrderBy(GenP((bm, chunks), forward, backward)).TileBy([bm, chunks])
+
+
+def lds_b_layout(bk, bn):
+    """B tile in elements, rows of ``bn``: ``k*bn + (n ^ 32*(k % 4))``.
+
+    A transposing read touches four consecutive k-rows, 64 bytes of each; rotating the
+    64-byte chunk index by ``k % 4`` puts the four rows on four different quarters of the
+    banks.  Bits 0-4 of ``n`` are untouched, so 16-byte stores and 8-byte reads stay whole."""
+    def key(k):
+        return (k % 4) * 32
+
+    def forward(kn):
+        k, n = kn
+        return k * bn + BitXor(sp.sympify(n), sp.sympify(key(k)))
+
+    def backward(flat):
+        k, p = flat // bn, flat % bn
+        return (k, BitXor(sp.sympify(p), sp.sympify(key(k))))
+
+    return OrderBy(GenP((bk, bn), forward, backward)).TileBy([bk, bn])
+
+
+def launch_order(num_pid_m, num_pid_n, group_m, pid):
+    """``(pid_m, pid_n)`` of the grouped launch order (matmul_sympy.py:57-65)."""
+    lay = OrderBy(Col(sp.Max(num_pid_m // group_m, 1), 1),
+                  Col(sp.Min(num_pid_m, group_m), num_pid_n)).TileBy([num_pid_m, num_pid_n])
+    return lay.inv(pid)
+
+
+def xcd_remap(per, wg, xcds=XCDS):
+    """Workgroup id -> position in the launch order such that the ids one XCD receives
+    (``wg % xcds`` is constant) form a contiguous run of ``per`` positions: read ``wg`` as
+    ``(j, x)`` of a row-major ``[per, xcds]`` box and store it column-major."""
+    j, x = OrderBy(Row(per, xcds)).TileBy([per, xcds]).inv(wg)
+    return OrderBy(Col(per, xcds)).TileBy([per, xcds])[j, x]
+
+
+def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
+    WAVES_M, WAVES_N = waves
+    THREADS = 64 * WAVES_M * WAVES_N
+    WM, WN = bm // WAVES_M, bn // WAVES_N
+    TM, TN = WM // 32, WN // 32
+    A_ITERS = bm * bk // 8 // THREADS
+    B_ITERS = bk * bn // 8 // THREADS
+    assert bm * bk // 8 % THREADS == 0 and bk * bn // 8 % THREADS == 0 and bk % 16 == 0
+
+    M, N, K = size("M"), size("N"), size("K")
+    npm, npn, per_xcd, group_m = size("num_pid_m"), size("num_pid_n"), size("wg_per_xcd"), size("GM")
+    t, it, wave, wg, pid, k, ks = (idx(n) for n in ("t", "it", "wave", "wg", "pid", "k", "ks"))
+    pid_m, pid_n = idx("pid_m"), idx("pid_n")
+    row, ch, kr = idx("row"), idx("ch"), idx("kr")
+    i, j, r = idx("i"), idx("j"), idx("r")
+    wm, wn, l32, lhi, l16, lgrp = (idx(n) for n in ("wm", "wn", "l32", "lhi", "l16", "lgrp"))
+    cr, cc = idx("cr"), idx("cc")
+
+    A_L = OrderBy(Row(M, K)).TileBy([M / bm, K / bk], [bm, bk])
+    B_L = OrderBy(Row(K, N)).TileBy([K / bk, N / bn], [bk, bn])
+    C_L = OrderBy(Row(M, N)).TileBy([M / bm, N / bn], [bm, bn])
+    As_L = lds_a_layout(bm, bk // 8)
+    Bs_L = lds_b_layout(bk, bn)
+
+    lane_rng = {t: (0, THREADS), it: (0, max(A_ITERS, B_ITERS))}
+    a_row, a_ch = (tidy(e, lane_rng) for e in
+                   OrderBy(Row(bm, bk // 8)).TileBy([bm, bk // 8]).inv(it * THREADS + t))
+    b_kr, b_ch = (tidy(e, lane_rng) for e in
+                  OrderBy(Row(bk, bn // 8)).TileBy([bk, bn // 8]).inv(it * THREADS + t))
+    wm_e, wn_e = OrderBy(Row(WAVES_M, WAVES_N)).TileBy([WAVES_M, WAVES_N]).inv(wave)
+
+    rng = {row: (0, bm), ch: (0, bk // 8), kr: (0, bk), i: (0, TM), j: (0, TN), r: (0, 16),
+           wm: (0, WAVES_M), wn: (0, WAVES_N), l32: (0, 32), lhi: (0, 2), l16: (0, 16),
+           lgrp: (0, 4), ks: (0, bk // 16), cr: (0, bm), cc: (0, bn), pid_m: (0, M / bm),
+           pid_n: (0, N / bn), k: (0, K / bk)}
+
+    frag_row = wm * WM + i * 32 + l32
+    frag_k = [ks * 16 + (lgrp // 2) * 8 + h * 4 + l16 // 4 for h in (0, 1)]
+    frag_n = wn * WN + j * 32 + (lgrp % 2) * 16 + 4 * (l16 % 4)
+    pm_e, pn_e = launch_order(npm, npn, group_m, pid)
+
+    params = dict(
+        banner=BANNER, BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
+        WM=WM, WN=WN, TM=TM, TN=TN, A_ITERS=A_ITERS, B_ITERS=B_ITERS, XCDS=XCDS, MAX_GROUPS=MAX_GROUPS,
+        pid_layout="OrderBy(Col(max(npm//GM,1),1), Col(min(npm,GM),npn)).TileBy([npm,npn]).inv(pid)",
+        MAX_GM=max_group_m,
+        xcd_layout=f"OrderBy(Col(nwg/{XCDS}, {XCDS})).TileBy([nwg/{XCDS}, {XCDS}])[Row(nwg/{XCDS}, {XCDS}).inv(wg)]",
+        a_layout=f"OrderBy(Row(M,K)).TileBy([M/{bm},K/{bk}],[{bm},{bk}])",
+        b_layout=f"OrderBy(Row(K,N)).TileBy([K/{bk},N/{bn}],[{bk},{bn}])",
+        c_layout=f"OrderBy(Row(M,N)).TileBy([M/{bm},N/{bn}],[{bm},{bn}])",
+        wm=code(wm_e), wn=code(wn_e),
+        a_row=code(a_row), a_ch=code(a_ch), b_kr=code(b_kr), b_ch=code(b_ch),
+        a_goff=code(tidy(A_L[pid_m, k, row, ch * 8], rng)),
+        b_goff=code(tidy(B_L[k, pid_n, kr, ch * 8], rng)),
+        a_loff=code(tidy(8 * As_L[row, ch], rng)),
+        b_loff=code(tidy(Bs_L[kr, ch * 8], rng)),
+        a_frag=code(tidy(8 * As_L[frag_row, ks * 2 + lhi], rng)),
+        b_frag0=code(tidy(Bs_L[frag_k[0], frag_n], rng)),
+        b_frag1=code(tidy(Bs_L[frag_k[1], frag_n], rng)),
+        c_row=code(wm * WM + i * 32 + (r // 4) * 8 + lhi * 4 + r % 4),
+        c_col=code(wn * WN + j * 32 + l32),
+        c_goff=code(tidy(C_L[pid_m, pid_n, cr, cc], rng)),
+        xcd_pid=code(tidy(xcd_remap(per_xcd, wg), {wg: (0, per_xcd * XCDS)})),
+        pid_m=code(pm_e), pid_n=code(pn_e),
+    )
+    text = template("gemm.hip.j2").render(**params)
+    meta = dict(BM=bm, BN=bn, BK=bk, MAX_GROUPS=MAX_GROUPS)
+    return Emitted("gemm_f16.hip", text, ["lego_gemm_f16_launch", "lego_grouped_gemm_f16_launch"]), meta

@@ -1,0 +1,114 @@
+"""Generator of the vectorised, LDS-staged transpose.
+
+The reference states a transpose as "copy every logical index from a row-major tiled
+layout to the column-major layout with the same tiling", decoding the block id row-major
+for reads and column-major for writes so that both sides are contiguous
+(benchmarks/mlir/transpose_smem.py:28-80).  This generator keeps that statement -- the
+source, destination and staging tiles are LEGO layouts and every address in the kernel is
+printed from them -- and changes what a lane moves: one 16-byte vector per access instead
+of one element, through a staging tile that is stored transposed with an XOR rotation
+instead of the reference's conflicting 32x32 array.
+
+Layouts (``R x C`` matrix, LEGO tiles ``TR x TC``, a workgroup owns ``MR x MC`` tiles):
+
+* source       ``OrderBy(Row(R, C)).TileBy([R/SR, C/SC], [MR, MC], [TR, TC])``
+* destination  ``OrderBy(Col(R, C)).TileBy(...same levels...)``
+* staging      ``OrderBy(GenP((KD, SR), swizzle)).TileBy([KD, SR])`` in 4-byte words, where
+  word-column ``k`` of row ``r`` holds source columns ``k`` (fp32) or ``2k, 2k+1`` (fp16).
+"""
+from __future__ import annotations
+
+import sympy as sp
+
+from ..lego import BitXor, Col, GenP, OrderBy, Row
+from .common import BANNER, Emitted, code, idx, size, template, tidy
+
+THREADS = 256
+
+
+def staging_key(k, sr, esize):
+    """XOR key of word-column ``k`` (a multiple of 4, so 16-byte row groups stay whole).
+
+    fp32: sixteen lanes of a wave write word-columns ``4*cv + e`` of four consecutive rows;
+    rotating the row digit by ``4*(k//4)`` sends them to 64 different banks, and the
+    sixteen 16-byte reads of one column in phase 2 cover all 64 banks once.
+    fp16: eight lanes cover one row, eight rows per instruction; ``8*(k//4)`` separates the
+    lanes of a row and ``4*(k%2)`` separates the two word-columns that share a 16-lane
+    read group in phase 2.
+    """
+    if esize == 4:
+        return ((k // 4) % (sr // 4)) * 4
+    return ((k // 4) % (sr // 8)) * 8 + (k % 2) * 4
+
+
+def staging_layout(kd, sr, esize):
+    def forward(kr):
+        k, r = kr
+        return k * sr + BitXor(sp.sympify(r), sp.sympify(staging_key(k, sr, esize)))
+
+    def backward(flat):
+        k, p = flat // sr, flat % sr
+        return (k, BitXor(sp.sympify(p), sp.sympify(staging_key(k, sr, esize))))
+
+    return OrderBy(GenP((kd, sr), forward, backward)).TileBy([kd, sr])
+
+
+def emit(dtype="f32", tile=(32, 32), group=(2, 2)):
+    """HIP translation unit for one element type and one tiling."""
+    elt, esize = {"f32": ("float", 4), "f16": ("_Float16", 2)}[dtype]
+    vec = 16 // esize                       # elements per 16-byte vector
+    (TR, TC), (MR, MC) = tile, group
+    SR, SC = MR * TR, MC * TC               # macro tile of a workgroup, in elements
+    KD = SC * esize // 4                    # word-columns of the staging tile
+    rows_per_read = 16 // 4 if esize == 4 else 8
+    assert (SR * SC) % (vec * THREADS) == 0 and SR % rows_per_read == 0
+    P1 = SR * SC // (vec * THREADS)
+    P2 = KD * (SR // rows_per_read) // THREADS
+    assert P2 >= 1 and KD * (SR // rows_per_read) % THREADS == 0
+
+    R, C = size("R"), size("C")
+    wg, t, it, e = idx("wg"), idx("t"), idx("it"), idx("e")
+    r, cv, k, rv = idx("r"), idx("cv"), idx("k"), idx("rv")
+    Bi, Bj = idx("Bi"), idx("Bj")
+    levels = ([R / SR, C / SC], [MR, MC], [TR, TC])
+    src = OrderBy(Row(R, C)).TileBy(*levels)
+    dst = OrderBy(Col(R, C)).TileBy(*levels)
+    lds = staging_layout(KD, SR, esize)
+
+    def in_tile(layout, row, col, ranges):
+        off = layout[Bi, Bj, row // TR, col // TC, row % TR, col % TC]
+        return tidy(off, ranges)
+
+    # workgroup -> macro tile, row-major over the grid of macro tiles
+    nBi, nBj = size("nBi"), size("nBj")
+    Bi_e, Bj_e = OrderBy(Row(nBi, nBj)).TileBy([nBi, nBj]).inv(wg)
+    # lane -> vector of the macro tile, phase 1: SC/vec vectors per row
+    v1 = OrderBy(Row(SR, SC // vec)).TileBy([SR, SC // vec]).inv(it * THREADS + t)
+    v1 = [tidy(x, {t: (0, THREADS), it: (0, P1)}) for x in v1]
+    # lane -> (word-column, row group), phase 2
+    v2 = OrderBy(Row(KD, SR // rows_per_read)).TileBy([KD, SR // rows_per_read]).inv(it * THREADS + t)
+    v2 = [tidy(x, {t: (0, THREADS), it: (0, P2)}) for x in v2]
+
+    rng1 = {r: (0, SR), cv: (0, SC // vec), e: (0, 4)}
+    rng2 = {k: (0, KD), rv: (0, SR // rows_per_read)}
+    cols_per_word = 4 // esize
+    params = dict(
+        banner=BANNER, elt=elt, esize=esize, SR=SR, SC=SC, KD=KD, THREADS=THREADS, P1=P1, P2=P2,
+        kernel=f"lego_transpose_{dtype}_{SR}x{SC}",
+        src_layout=f"OrderBy(Row(R, C)).TileBy([R/{SR}, C/{SC}], [{MR}, {MC}], [{TR}, {TC}])",
+        dst_layout=f"OrderBy(Col(R, C)).TileBy([R/{SR}, C/{SC}], [{MR}, {MC}], [{TR}, {TC}])",
+        lds_layout=f"OrderBy(GenP(({KD}, {SR}), xor-rotated rows)).TileBy([{KD}, {SR}])",
+        Bi=code(Bi_e), Bj=code(Bj_e),
+        p1_r=code(v1[0]), p1_cv=code(v1[1]),
+        src_off=code(in_tile(src, r, cv * vec, rng1)),
+        lds_store=code(tidy(lds[cv * 4 + e, r], rng1)),
+        p2_k=code(v2[0]), p2_rv=code(v2[1]),
+        lds_load0=code(tidy(lds[k, rv * rows_per_read], rng2)),
+        lds_load1=code(tidy(lds[k, rv * rows_per_read + 4], rng2)) if esize == 2 else "",
+        dst_off0=code(in_tile(dst, rv * rows_per_read, k * cols_per_word, rng2)),
+        dst_off1=code(in_tile(dst, rv * rows_per_read, k * cols_per_word + 1, rng2)) if esize == 2 else "",
+        grid=f"static_cast<unsigned>(rows / {SR}) * static_cast<unsigned>(cols / {SC})",
+    )
+    text = template("transpose.hip.j2").render(**params)
+    return Emitted(f"transpose_{dtype}.hip", text, [params["kernel"] + "_launch"]), dict(
+        SR=SR, SC=SC, kernel=params["kernel"])

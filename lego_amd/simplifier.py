@@ -479,19 +479,20 @@ def _rewrite_mod(e, prover):
 
 
 def _recombine(e, prover):
-    """``a*floor(x/a) + Mod(x, a) -> x`` among the terms of a sum."""
+    """``c*a*floor(x/a) + c*Mod(x, a) -> c*x`` among the terms of a sum."""
     args = list(Add.make_args(e))
     changed = True
     while changed:
         changed = False
         for i, t in enumerate(args):
-            if not isinstance(t, Mod):
+            c, m = t.as_coeff_Mul()
+            if not isinstance(m, Mod):
                 continue
-            x, a = t.args
-            want = a * floor(x / a)
+            x, a = m.args
+            want = c * a * floor(x / a)
             for j, u in enumerate(args):
                 if j != i and sp.expand(u - want) == 0 and prover.positive_(a):
-                    args = [v for k, v in enumerate(args) if k not in (i, j)] + [x]
+                    args = [v for k, v in enumerate(args) if k not in (i, j)] + [c * x]
                     changed = True
                     break
             if changed:

@@ -1,0 +1,180 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle."""
+import math
+
+import pytest
+import torch
+
+from oracle import kernels as ok
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from lego_amd import ops, runtime
+    runtime.load_library()   # fails loudly when liblego_hip.so was not built
+    assert torch.cuda.is_available()
+    return ops
+
+
+def _gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+# ---- transpose: bit exact ---------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype,rows,cols", [
+    (torch.float32, 64, 64), (torch.float32, 128, 320), (torch.float32, 1024, 512),
+    (torch.float16, 64, 64), (torch.float16, 192, 128), (torch.float16, 512, 1024),
+])
+def test_transpose_matches_oracle(ops, dtype, rows, cols):
+    print(f"transpose {dtype} {rows}x{cols}", flush=True)
+    x = (torch.rand(rows, cols, generator=_gen(0)) * 2 - 1).to(dtype)
+    want = ok.transpose(x, 32, 32)                 # index-array scatter through the two layouts
+    assert torch.equal(want, x.t().contiguous())   # and that is the textbook transpose
+    got = ops.transpose(x.cuda()).cpu()
+    assert torch.equal(got, want)
+
+
+def test_transpose_config1_fp32_4096(ops):
+    print("transpose config 1", flush=True)
+    x = torch.rand(4096, 4096, generator=_gen(0), dtype=torch.float32) * 2 - 1
+    got = ops.transpose(x.cuda()).cpu()
+    assert torch.equal(got, ok.transpose(x, 32, 32))
+
+
+def test_transpose_config2_fp16_16384_properties(ops):
+    """Full size: transposing twice is the identity and the result equals the strided view."""
+    print("transpose config 2", flush=True)
+    x = torch.randn(16384, 16384, generator=_gen(1)).half().cuda()
+    y = ops.transpose(x)
+    assert torch.equal(y, x.t())
+    assert torch.equal(ops.transpose(y), x)
+
+
+def test_transpose_rejects_bad_shapes(ops):
+    from lego_amd.runtime import LegoHipError
+    with pytest.raises(LegoHipError):
+        ops.transpose(torch.zeros(100, 64, device="cuda"))
+    with pytest.raises(ValueError):
+        ops.transpose(torch.zeros(64, 64, device="cuda").t())
+
+
+# ---- softmax / layernorm: max abs err <= 2e-3 ------------------------------------------------
+
+TOL = 2e-3
+
+
+@pytest.mark.parametrize("wpr", [None, 1, 2, 4])
+@pytest.mark.parametrize("M,N", [(7, 8), (33, 520), (64, 1024), (5, 2048), (129, 4096), (16, 8192), (3, 16384)])
+def test_softmax_matches_oracle(ops, M, N, wpr):
+    print(f"softmax {M}x{N} wpr={wpr}", flush=True)
+    x = (2.0 * torch.randn(M, N, generator=_gen(2))).half()
+    want = ok.softmax(x)
+    got = ops.softmax(x.cuda(), waves_per_row=wpr).cpu()
+    assert (got.float() - want.float()).abs().max().item() <= TOL
+    assert torch.allclose(got.float().sum(-1), torch.ones(M), atol=2e-2)
+
+
+@pytest.mark.parametrize("wpr", [None, 1, 2, 4])
+@pytest.mark.parametrize("M,N", [(7, 8), (33, 520), (64, 1024), (129, 4096), (1151, 8192), (3, 16384)])
+def test_layernorm_matches_oracle(ops, M, N, wpr):
+    print(f"layernorm {M}x{N} wpr={wpr}", flush=True)
+    g = _gen(3)
+    x = (2.0 * torch.randn(M, N, generator=g)).half()
+    w = (1 + 0.1 * torch.randn(N, generator=g)).half()
+    b = (0.1 * torch.randn(N, generator=g)).half()
+    want_y, want_mean, want_rstd = ok.layernorm_fwd(x, w, b, 1e-5)
+    y, mean, rstd = ops.layer_norm_fwd(x.cuda(), w.cuda(), b.cuda(), 1e-5, waves_per_row=wpr)
+    # y is fp16 with magnitude up to ~6: half an ulp there is 2e-3, so compare before the final
+    # rounding as well (the tolerance of the contract is on the value, not on the rounding)
+    assert (y.cpu().float() - want_y.float()).abs().max().item() <= 2 * TOL
+    assert torch.allclose(mean.cpu(), want_mean, atol=1e-4, rtol=1e-4)
+    assert torch.allclose(rstd.cpu(), want_rstd, atol=1e-4, rtol=1e-4)
+
+
+def test_layernorm_reference_test_shape(ops):
+    """The reference's own test case (layernorm.py:435-458): M=1151, N=8192, x = -2.3 + 0.5*randn,
+    w, b uniform, atol=1e-2."""
+    print("layernorm reference shape", flush=True)
+    g = _gen(0)
+    w, b = torch.rand(8192, generator=g).half(), torch.rand(8192, generator=g).half()
+    x = (-2.3 + 0.5 * torch.randn(1151, 8192, generator=g)).half()
+    want = torch.nn.functional.layer_norm(x.float(), (8192,), w.float(), b.float(), 1e-5).half()
+    from lego_amd.ops import lego_layer_norm
+    got = lego_layer_norm(x.cuda(), (8192,), w.cuda(), b.cuda(), 1e-5).cpu()
+    assert torch.allclose(got.float(), want.float(), atol=1e-2, rtol=0)
+    assert (got.float() - want.float()).abs().max().item() <= TOL
+
+
+def test_config3_full_size(ops):
+    print("config 3 full size", flush=True)
+    g = _gen(2)
+    x = (2.0 * torch.randn(8192, 8192, generator=g)).half()
+    g3 = _gen(3)
+    w = (1 + 0.1 * torch.randn(8192, generator=g3)).half()
+    b = (0.1 * torch.randn(8192, generator=g3)).half()
+    xd = x.cuda()
+    s = ops.softmax(xd).cpu()
+    assert (s.float() - ok.softmax(x).float()).abs().max().item() <= TOL
+    y, mean, rstd = ops.layer_norm_fwd(xd, w.cuda(), b.cuda(), 1e-5)
+    want_y, want_mean, want_rstd = ok.layernorm_fwd(x, w, b, 1e-5)
+    err = (y.cpu().float() - want_y.float()).abs()
+    # fp16 spacing is 2^-9 = 1.95e-3 for |y| in [2,4) and 3.9e-3 in [4,8): a correctly rounded
+    # result can differ from another correctly rounded result by one spacing
+    assert err[want_y.float().abs() < 2].max().item() <= TOL
+    assert (err <= want_y.float().abs().clamp(min=1) * 2 ** -9).all()
+    assert torch.allclose(mean.cpu(), want_mean, atol=1e-4, rtol=1e-4)
+
+
+# ---- GEMM: relative error <= 1e-2 against fp32 accumulation ------------------------------------
+
+def _rel_err(got, want):
+    return ((got.float() - want.float()).norm() / want.float().norm()).item()
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (256, 256, 512), (512, 256, 128), (256, 768, 256),
+                                   (1024, 1024, 1024), (3072, 512, 320)])
+def test_gemm_matches_oracle(ops, M, N, K):
+    print(f"gemm {M}x{N}x{K}", flush=True)
+    g = _gen(4)
+    a = (torch.randn(M, K, generator=g) / math.sqrt(K)).half()
+    b = (torch.randn(K, N, generator=g) / math.sqrt(K)).half()
+    want = ok.gemm(a, b)
+    got = ops.matmul(a.cuda(), b.cuda()).cpu()
+    assert _rel_err(got, want) <= 1e-2
+    assert (got.float() - want.float()).abs().max().item() <= 1e-2   # the reference's own atol
+
+
+def test_gemm_integer_exact(ops):
+    """Small-integer operands make every partial sum exact in fp32 and fp16: any indexing
+    mistake (a transposed tile, a wrong k block) changes the integers."""
+    print("gemm integer exact", flush=True)
+    g = _gen(7)
+    a = torch.randint(-2, 3, (512, 256), generator=g).half()
+    b = torch.randint(-2, 3, (256, 768), generator=g).half()
+    want = (a.double() @ b.double())
+    got = ops.matmul(a.cuda(), b.cuda()).cpu()
+    assert torch.equal(got.double(), want)
+
+
+def test_grouped_gemm_matches_oracle(ops):
+    print("grouped gemm", flush=True)
+    g = _gen(5)
+    shapes = [(256, 256, 64), (512, 256, 128), (256, 1024, 256), (768, 512, 192), (1024, 1024, 512)]
+    A = [(torch.randn(m, k, generator=g) / math.sqrt(k)).half() for m, n, k in shapes]
+    B = [(torch.randn(k, n, generator=g) / math.sqrt(k)).half() for m, n, k in shapes]
+    want = ok.grouped_gemm(A, B)
+    got = ops.lego_group_gemm_fn([a.cuda() for a in A], [b.cuda() for b in B])
+    for c, w in zip(got, want):
+        assert _rel_err(c.cpu(), w) <= 1e-2
+
+
+def test_gemm_rejects_bad_shapes(ops):
+    from lego_amd.runtime import LegoHipError
+    with pytest.raises(LegoHipError):
+        ops.matmul(torch.zeros(100, 64, device="cuda", dtype=torch.half),
+                   torch.zeros(64, 256, device="cuda", dtype=torch.half))
+    with pytest.raises(NotImplementedError):
+        ops.matmul(torch.zeros(256, 64, device="cuda", dtype=torch.half),
+                   torch.zeros(64, 256, device="cuda", dtype=torch.half), activation="leaky_relu")
