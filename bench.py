@@ -1,0 +1,245 @@
+#!/usr/bin/env python3
+"""Benchmark of the lego_hip hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  A "step" is one launch of the headline workload, the fp16
+16384x16384 transpose through the LEGO tiled + XOR-swizzled staging layout (the second
+configuration of BASELINE.json); ``value`` is its effective HBM bandwidth with the input
+already resident in device memory.  The other four configurations are timed in the same
+run with the same K and W and reported under ``kernels`` with their own roofline
+fractions.  ``cpu_baseline`` times the CPU oracle (index arrays through the two layouts +
+gather/scatter) on a bounded panel of the same matrix, on this host's cores.
+
+Timing uses HIP events recorded on the stream the kernels are launched on (torch's
+current stream).  Working sets that fit the 256 MB Infinity Cache are timed twice: "hot"
+(same buffers every launch) and "rotating" (a pool of buffers larger than the cache).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
+
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/transpose_f16_16384_pmc.txt); None until measured.
+HEADLINE_TRAFFIC_BYTES = None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="comma list of configs to time (c1,c2,c3,c4,c5)")
+    ns = ap.parse_args()
+    if ns.gpus != 1:
+        print("bench.py: this build measures one MI355X; every configuration of the hot path is a "
+              "single-GPU kernel and --gpus above 1 is not supported", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from lego_amd import ops, runtime
+    runtime.load_library()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    K, W = ns.steps, ns.warmup
+    only = set(filter(None, ns.only.split(",")))
+
+    def want(name):
+        return not only or name in only
+
+    def timed(fn, steps=K, warmup=W):
+        """Average milliseconds per call over ``steps`` calls, bracketed by synchronisation."""
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(steps):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / steps
+
+    def rotating(make, call, pool_bytes, each_bytes):
+        """Time ``call(buffers)`` cycling through enough buffer sets to exceed the cache."""
+        n = max(2, math.ceil(pool_bytes / each_bytes))
+        sets = [make() for _ in range(n)]
+        state = {"i": 0}
+
+        def fn():
+            call(sets[state["i"] % n])
+            state["i"] += 1
+        return timed(fn)
+
+    kernels = {}
+    gen = lambda seed: torch.Generator().manual_seed(seed)  # noqa: E731
+
+    # ---- C2 (headline): fp16 16384^2 transpose ------------------------------------------
+    n2 = 16384
+    x2 = torch.randn(n2, n2, generator=gen(1)).half().to(dev)
+    out2 = ops.transpose(x2)
+    assert torch.equal(out2, x2.t()), "transpose parity failed"
+    bytes2 = 2 * n2 * n2 * 2
+    y2 = torch.empty_like(x2)
+    # the timed region calls the C ABI directly on preallocated buffers
+    import ctypes
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+
+    def c2():
+        runtime.call("lego_hip_transpose_f16", p(x2), p(y2), n2, n2, stream)
+    ms2 = timed(c2)
+    gbs2 = bytes2 / ms2 / 1e6
+    copy_ms = timed(lambda: y2.copy_(x2))
+    copy_gbs = bytes2 / copy_ms / 1e6
+    kernels["c2_transpose_f16_16384"] = dict(ms=ms2, gbs=gbs2, frac_hbm=gbs2 / HBM_PEAK_GBS,
+                                             bytes=bytes2, parity="bit-exact")
+    kernels["device_copy_512MiB"] = dict(ms=copy_ms, gbs=copy_gbs, frac_hbm=copy_gbs / HBM_PEAK_GBS,
+                                         note="torch copy_ of the same buffers: achievable ceiling")
+
+    # ---- C1: fp32 4096^2 transpose ---------------------------------------------------------
+    if want("c1"):
+        n1 = 4096
+        x1 = (torch.rand(n1, n1, generator=gen(0), dtype=torch.float32) * 2 - 1).to(dev)
+        assert torch.equal(ops.transpose(x1), x1.t())
+        y1 = torch.empty_like(x1)
+        b1 = 2 * n1 * n1 * 4
+        hot = timed(lambda: runtime.call("lego_hip_transpose_f32", p(x1), p(y1), n1, n1, stream))
+        rot = rotating(lambda: (torch.rand(n1, n1, device=dev), torch.empty(n1, n1, device=dev)),
+                       lambda s: runtime.call("lego_hip_transpose_f32", p(s[0]), p(s[1]), n1, n1, stream),
+                       1 << 30, b1)
+        kernels["c1_transpose_f32_4096"] = dict(ms_hot=hot, gbs_hot=b1 / hot / 1e6, ms=rot, gbs=b1 / rot / 1e6,
+                                                frac_hbm=b1 / rot / 1e6 / HBM_PEAK_GBS, bytes=b1,
+                                                parity="bit-exact",
+                                                note="gbs = rotating buffers (1 GiB pool); gbs_hot = cache resident")
+        del x1, y1
+
+    # ---- C3: softmax and LayerNorm forward, fp16 8192x8192 -------------------------------------
+    if want("c3"):
+        m3 = n3 = 8192
+        x3c = (2.0 * torch.randn(m3, n3, generator=gen(2))).half()
+        g3 = gen(3)
+        w3c = (1 + 0.1 * torch.randn(n3, generator=g3)).half()
+        b3c = (0.1 * torch.randn(n3, generator=g3)).half()
+        x3, w3, b3 = x3c.to(dev), w3c.to(dev), b3c.to(dev)
+        y3 = torch.empty_like(x3)
+        mean3 = torch.empty(m3, device=dev)
+        rstd3 = torch.empty(m3, device=dev)
+        by3 = 2 * m3 * n3 * 2
+        ref_s = torch.softmax(x3.float(), -1)
+        err_s = (ops.softmax(x3).float() - ref_s).abs().max().item()
+        ref_l = torch.nn.functional.layer_norm(x3.float(), (n3,), w3.float(), b3.float(), 1e-5)
+        err_l = (ops.layer_norm_fwd(x3, w3, b3, 1e-5)[0].float() - ref_l).abs().max().item()
+        del ref_s, ref_l
+
+        def sm(s=None):
+            xx, yy = (x3, y3) if s is None else s
+            runtime.call("lego_hip_softmax_f16", p(xx), p(yy), m3, n3, stream)
+
+        def ln(s=None):
+            xx, yy = (x3, y3) if s is None else s
+            runtime.call("lego_hip_layernorm_fwd_f16", p(xx), p(yy), p(w3), p(b3), p(mean3), p(rstd3),
+                         m3, n3, ctypes.c_float(1e-5), stream)
+        mk = lambda: (x3.clone(), torch.empty_like(x3))  # noqa: E731
+        for name, fn, err in (("c3_softmax_f16_8192", sm, err_s), ("c3_layernorm_fwd_f16_8192", ln, err_l)):
+            hot = timed(fn)
+            rot = rotating(mk, fn, 1 << 30, by3)
+            kernels[name] = dict(ms_hot=hot, gbs_hot=by3 / hot / 1e6, ms=rot, gbs=by3 / rot / 1e6,
+                                 frac_hbm=by3 / rot / 1e6 / HBM_PEAK_GBS, bytes=by3, max_abs_err_vs_fp32=err,
+                                 note="gbs = rotating buffers (1 GiB pool); gbs_hot = cache resident; "
+                                      "x ~ N(0, sigma=2)")
+        del x3, y3
+
+    # ---- C4: fp16 GEMM 8192^3 ----------------------------------------------------------------------
+    if want("c4"):
+        n4 = 8192
+        g4 = gen(4)
+        a4 = (torch.randn(n4, n4, generator=g4) / math.sqrt(n4)).half().to(dev)
+        b4 = (torch.randn(n4, n4, generator=g4) / math.sqrt(n4)).half().to(dev)
+        c4 = torch.empty(n4, n4, dtype=torch.half, device=dev)
+        fl4 = 2 * n4 ** 3
+
+        def gm():
+            runtime.call("lego_hip_gemm_f16", p(a4), p(b4), p(c4), n4, n4, n4, stream)
+        gm()
+        # parity on a 512-row panel against fp32 accumulation
+        ref = a4[:512].float() @ b4.float()
+        rel = ((c4[:512].float() - ref).norm() / ref.norm()).item()
+        ms = timed(gm, steps=max(5, K // 5), warmup=max(2, W // 5))
+        lib_ms = timed(lambda: torch.matmul(a4, b4, out=c4), steps=max(5, K // 5), warmup=max(2, W // 5))
+        kernels["c4_gemm_f16_8192"] = dict(ms=ms, tflops=fl4 / ms / 1e9, frac_mfma=fl4 / ms / 1e9 / MFMA_F16_PEAK_TFLOPS,
+                                           flop=fl4, rel_err_vs_fp32=rel,
+                                           vendor_library_tflops=fl4 / lib_ms / 1e9,
+                                           note="vendor_library = torch.matmul (hipBLASLt) on the same buffers")
+        del a4, b4, c4, ref
+
+    # ---- C5: grouped fp16 GEMM, 8 problems -------------------------------------------------------------
+    if want("c5"):
+        g5 = gen(5)
+        idx = torch.randint(0, 3, (8, 3), generator=g5)
+        dims = [[(1024, 2048, 4096)[int(v)] for v in row] for row in idx]
+        A = [(torch.randn(m, k, generator=g5) / math.sqrt(k)).half().to(dev) for m, n, k in dims]
+        B = [(torch.randn(k, n, generator=g5) / math.sqrt(k)).half().to(dev) for m, n, k in dims]
+        C = [torch.empty(m, n, dtype=torch.half, device=dev) for m, n, k in dims]
+        arr = ctypes.c_void_p * 8
+        pa, pb, pc = arr(*[t.data_ptr() for t in A]), arr(*[t.data_ptr() for t in B]), arr(*[t.data_ptr() for t in C])
+        sz = (ctypes.c_int * 24)(*[v for d in dims for v in d])
+
+        def gg():
+            runtime.call("lego_hip_grouped_gemm_f16", pa, pb, pc, sz, 8, stream)
+        gg()
+        rel = max(((c.float() - a.float() @ b.float()).norm() / (a.float() @ b.float()).norm()).item()
+                  for a, b, c in zip(A, B, C))
+        fl5 = sum(2 * m * n * k for m, n, k in dims)
+        ms = timed(gg, steps=max(5, K // 5), warmup=max(2, W // 5))
+        kernels["c5_grouped_gemm_f16"] = dict(ms=ms, tflops=fl5 / ms / 1e9, frac_mfma=fl5 / ms / 1e9 / MFMA_F16_PEAK_TFLOPS,
+                                              flop=fl5, problems=dims, rel_err_vs_fp32=rel)
+        del A, B, C
+
+    # ---- CPU baseline: the oracle on a bounded panel of the headline matrix ------------------------------
+    cpu = None
+    if not ns.skip_cpu:
+        from oracle import kernels as ok
+        rows = 2048
+        c2()                      # y2 was last written by the copy ceiling measurement
+        torch.cuda.synchronize()
+        panel = x2[:rows].cpu()
+        torch.set_num_threads(min(16, os.cpu_count() or 1))
+        t0 = time.perf_counter()
+        got = ok.transpose(panel, 64, 64)
+        dt = time.perf_counter() - t0
+        assert torch.equal(got, y2[:, :rows].cpu()), "GPU result differs from the CPU oracle"
+        cpu = dict(value=2 * panel.numel() * 2 / dt / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                   sample=f"rows 0..{rows - 1} of the 16384x16384 fp16 matrix ({rows}x16384 panel, 1/8 of the "
+                          f"workload): offsets of both LEGO layouts evaluated with numpy, then one gather/scatter; "
+                          f"{dt:.2f} s on {os.cpu_count()} visible cores")
+
+    line = {
+        "metric": "HBM GB/s (transpose/softmax/LN) + fp16 GEMM TFLOPS, % of roofline, 1 GPU",
+        "value": gbs2, "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": ms2,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "2-D fp16 transpose 16384x16384, LEGO TileBy([256,256],[64,64]) row-major -> "
+                               "column-major with XOR-swizzled LDS staging, inputs N(0,1) seed 1"},
+        "roofline": {"bound": "hbm", "achieved": gbs2, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": gbs2 / HBM_PEAK_GBS, "traffic": HEADLINE_TRAFFIC_BYTES,
+                     "kernel": "lego_transpose_f16_64x64", "algorithmic_bytes_per_launch": bytes2},
+        "cpu_baseline": cpu,
+        "kernels": kernels,
+        "peaks": {"hbm_gbs": HBM_PEAK_GBS, "mfma_f16_tflops": MFMA_F16_PEAK_TFLOPS},
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
