@@ -93,7 +93,7 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
     t, it, wave, wg, pid, k, ks = (idx(n) for n in ("t", "it", "wave", "wg", "pid", "k", "ks"))
     pid_m, pid_n = idx("pid_m"), idx("pid_n")
     row, ch, kr = idx("row"), idx("ch"), idx("kr")
-    i, j, r = idx("i"), idx("j"), idx("r")
+    i, j, r, q = idx("i"), idx("j"), idx("r"), idx("q")
     wm, wn, l32, lhi, l16, lgrp = (idx(n) for n in ("wm", "wn", "l32", "lhi", "l16", "lgrp"))
     cr, cc = idx("cr"), idx("cc")
 
@@ -115,10 +115,35 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
            lgrp: (0, 4), ks: (0, bk // 16), cr: (0, bm), cc: (0, bn), pid_m: (0, M / bm),
            pid_n: (0, N / bn), k: (0, K / bk)}
 
+    def chunk_walk(expr, n_iters):
+        """``expr`` (a function of the lane ``t`` and the chunk counter ``it``) as
+        ``expr(it=0) + it*step`` with a lane-independent ``step``; raises if it is not."""
+        at = [tidy(sp.sympify(expr).subs(it, v), {t: (0, THREADS)}) for v in range(n_iters)]
+        step = sp.simplify(at[1] - at[0]) if n_iters > 1 else sp.Integer(0)
+        if t in step.free_symbols:
+            raise ValueError(f"chunk stride depends on the lane: {step}")
+        for v in range(n_iters):   # exhaustive over lanes: the walk really is affine
+            for lane in range(THREADS):
+                if (at[v] - at[0] - v * step).subs(t, lane) != 0:
+                    raise ValueError("chunk offsets are not affine in the chunk counter")
+        return at[0], step
+
     frag_row = wm * WM + i * 32 + l32
     frag_k = [ks * 16 + (lgrp // 2) * 8 + h * 4 + l16 // 4 for h in (0, 1)]
     frag_n = wn * WN + j * 32 + (lgrp % 2) * 16 + 4 * (l16 % 4)
     pm_e, pn_e = launch_order(npm, npn, group_m, pid)
+
+    sub_a = {row: a_row, ch: a_ch}
+    sub_b = {kr: b_kr, ch: b_ch}
+    a_full = tidy(A_L[pid_m, k, row, ch * 8], rng)     # the reference's a_ptrs expression
+    b_full = tidy(B_L[k, pid_n, kr, ch * 8], rng)     # and its b_ptrs expression
+    a_src0, a_src_step = chunk_walk(a_full.subs({pid_m: 0, k: 0}).subs(sub_a), A_ITERS)
+    b_src0, b_src_step = chunk_walk(b_full.subs({pid_n: 0, k: 0}).subs(sub_b), B_ITERS)
+    a_dst0, a_dst_step = chunk_walk(tidy(8 * As_L[row, ch], rng).subs(sub_a), A_ITERS)
+    b_dst0, b_dst_step = chunk_walk(tidy(Bs_L[kr, ch * 8], rng).subs(sub_b), B_ITERS)
+    chunk_params = dict(a_src0=code(a_src0), a_src_step=code(a_src_step), b_src0=code(b_src0),
+                        b_src_step=code(b_src_step), a_dst0=code(a_dst0), a_dst_step=code(a_dst_step),
+                        b_dst0=code(b_dst0), b_dst_step=code(b_dst_step))
 
     params = dict(
         banner=BANNER, BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
@@ -131,15 +156,19 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
         c_layout=f"OrderBy(Row(M,N)).TileBy([M/{bm},N/{bn}],[{bm},{bn}])",
         wm=code(wm_e), wn=code(wn_e),
         a_row=code(a_row), a_ch=code(a_ch), b_kr=code(b_kr), b_ch=code(b_ch),
-        a_goff=code(tidy(A_L[pid_m, k, row, ch * 8], rng)),
-        b_goff=code(tidy(B_L[k, pid_n, kr, ch * 8], rng)),
+        # offset of a chunk = tile base (uniform) + position inside k-tile 0 (per lane) + k * step
+        **chunk_params,
+        a_goff_base=code(a_full.subs({k: 0, row: 0, ch: 0})),
+        b_goff_base=code(b_full.subs({k: 0, kr: 0, ch: 0})),
+        a_kstep=code(sp.simplify(a_full.subs(k, k + 1) - a_full)),
+        b_kstep=code(sp.simplify(b_full.subs(k, k + 1) - b_full)),
         a_loff=code(tidy(8 * As_L[row, ch], rng)),
         b_loff=code(tidy(Bs_L[kr, ch * 8], rng)),
         a_frag=code(tidy(8 * As_L[frag_row, ks * 2 + lhi], rng)),
         b_frag0=code(tidy(Bs_L[frag_k[0], frag_n], rng)),
         b_frag1=code(tidy(Bs_L[frag_k[1], frag_n], rng)),
-        c_row=code(wm * WM + i * 32 + (r // 4) * 8 + lhi * 4 + r % 4),
-        c_col=code(wn * WN + j * 32 + l32),
+        c_row=code(wm * WM + i * 32 + l32),
+        c_col=code(wn * WN + j * 32 + q * 8 + lhi * 4),
         c_goff=code(tidy(C_L[pid_m, pid_n, cr, cc], rng)),
         xcd_pid=code(tidy(xcd_remap(per_xcd, wg), {wg: (0, per_xcd * XCDS)})),
         pid_m=code(pm_e), pid_n=code(pn_e),
