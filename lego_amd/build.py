@@ -24,8 +24,15 @@ LIB_PATH = LIB_DIR / "liblego_hip.so"
 OBJ_DIR = LIB_DIR / "obj"
 
 # the tilings the library is built with
-TRANSPOSE_F32 = dict(dtype="f32", tile=(32, 32), group=(2, 2))
-TRANSPOSE_F16 = dict(dtype="f16", tile=(64, 64), group=(1, 1))
+# Two tilings per element type: a wide macro tile (long read segments; fastest on MI355X) and a
+# 64x64 one for shapes the wide tile does not divide.  Tiles are dealt to workgroups in the
+# skewed ("diag") order.
+TRANSPOSE = {
+    "f32": [dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag"),
+            dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag")],
+    "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag"),
+            dict(dtype="f16", tile=(64, 64), group=(1, 1), order="diag")],
+}
 ROWWISE_WAVES = (1, 2, 4)
 ROWWISE_DEFAULT_WAVES = 4
 ROWWISE_MAX_N = 16384
@@ -35,20 +42,28 @@ GEMM = dict(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8)
 def generate():
     """Write every generated source; returns the list of .hip paths to compile."""
     units = []
-    t32, m32 = transpose.emit(**TRANSPOSE_F32)
-    t16, m16 = transpose.emit(**TRANSPOSE_F16)
-    units += [t32, t16]
+    tmeta = {}
+    for dtype, configs in TRANSPOSE.items():
+        for cfg in configs:
+            unit, meta = transpose.emit(**cfg, suffix="")
+            unit.filename = f"transpose_{dtype}_{meta['SR']}x{meta['SC']}.hip"
+            units.append(unit)
+            tmeta.setdefault(dtype, []).append(meta)
     units += [rowwise.emit(w) for w in ROWWISE_WAVES]
     g, mg = gemm.emit(**GEMM)
     units.append(g)
 
     h = [f"// {BANNER}", "#pragma once", "#include <hip/hip_runtime.h>", ""]
-    h += [f"hipError_t {m32['kernel']}_launch(const void*, void*, int, int, hipStream_t);",
-          f"hipError_t {m16['kernel']}_launch(const void*, void*, int, int, hipStream_t);",
-          f"#define LEGO_TRANSPOSE_F32_LAUNCH {m32['kernel']}_launch",
-          f"#define LEGO_TRANSPOSE_F32_SR {m32['SR']}", f"#define LEGO_TRANSPOSE_F32_SC {m32['SC']}",
-          f"#define LEGO_TRANSPOSE_F16_LAUNCH {m16['kernel']}_launch",
-          f"#define LEGO_TRANSPOSE_F16_SR {m16['SR']}", f"#define LEGO_TRANSPOSE_F16_SC {m16['SC']}", ""]
+    for dtype, metas in tmeta.items():
+        for m in metas:
+            h.append(f"hipError_t {m['kernel']}_launch(const void*, void*, int, int, hipStream_t);")
+        h += [f"// picks the first tiling that divides the shape; hipErrorInvalidValue if none does",
+              f"inline hipError_t lego_transpose_{dtype}_dispatch(const void* in, void* out, int rows, int cols, "
+              "hipStream_t stream) {"]
+        for m in metas:
+            h.append(f"  if (rows % {m['SR']} == 0 && cols % {m['SC']} == 0) "
+                     f"return {m['kernel']}_launch(in, out, rows, cols, stream);")
+        h += ["  return hipErrorInvalidValue;", "}", ""]
     for w in ROWWISE_WAVES:
         h += [f"hipError_t lego_softmax_f16_w{w}_launch(const void*, void*, int, int, hipStream_t);",
               f"hipError_t lego_layernorm_fwd_f16_w{w}_launch(const void*, void*, const void*, const void*, "

@@ -28,15 +28,15 @@ int lego_hip_abi_version(void) { return 1; }
 int lego_hip_transpose_f32(const void* in, void* out, int rows, int cols, void* stream)
 {
   if (!usable(in) || !usable(out) || in == out) return kInvalid;
-  if (rows <= 0 || cols <= 0 || rows % LEGO_TRANSPOSE_F32_SR || cols % LEGO_TRANSPOSE_F32_SC) return kInvalid;
-  return ok_or(LEGO_TRANSPOSE_F32_LAUNCH(in, out, rows, cols, as_stream(stream)));
+  if (rows <= 0 || cols <= 0) return kInvalid;
+  return ok_or(lego_transpose_f32_dispatch(in, out, rows, cols, as_stream(stream)));
 }
 
 int lego_hip_transpose_f16(const void* in, void* out, int rows, int cols, void* stream)
 {
   if (!usable(in) || !usable(out) || in == out) return kInvalid;
-  if (rows <= 0 || cols <= 0 || rows % LEGO_TRANSPOSE_F16_SR || cols % LEGO_TRANSPOSE_F16_SC) return kInvalid;
-  return ok_or(LEGO_TRANSPOSE_F16_LAUNCH(in, out, rows, cols, as_stream(stream)));
+  if (rows <= 0 || cols <= 0) return kInvalid;
+  return ok_or(lego_transpose_f16_dispatch(in, out, rows, cols, as_stream(stream)));
 }
 
 int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per_row, void* stream)

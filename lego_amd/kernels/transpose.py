@@ -53,7 +53,28 @@ def staging_layout(kd, sr, esize):
     return OrderBy(GenP((kd, sr), forward, backward)).TileBy([kd, sr])
 
 
-def emit(dtype="f32", tile=(32, 32), group=(2, 2)):
+def tile_order(order, n_bi, n_bj, wg):
+    """Workgroup id -> macro tile ``(Bi, Bj)``.
+
+    ``row``: tiles of one tile-row are consecutive (contiguous reads, strided writes);
+    ``col``: the transpose of that (strided reads, contiguous writes);
+    ``diag``: row order skewed by the tile row, ``Bj = (j + Bi) % n_bj``, so that workgroups
+    that run together spread both their reads and their writes over tile columns -- the
+    classic remedy for DRAM channel camping when the row pitch is a power of two.
+    """
+    if order == "row":
+        return OrderBy(Row(n_bi, n_bj)).TileBy([n_bi, n_bj]).inv(wg)
+    if order == "col":
+        return OrderBy(Col(n_bi, n_bj)).TileBy([n_bi, n_bj]).inv(wg)
+    if order == "diag":
+        skew = GenP((n_bi, n_bj),
+                    lambda ij: ij[0] * n_bj + (ij[1] - ij[0]) % n_bj,
+                    lambda f: (f // n_bj, (f % n_bj + f // n_bj) % n_bj))
+        return OrderBy(skew).TileBy([n_bi, n_bj]).inv(wg)
+    raise ValueError(order)
+
+
+def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix=""):
     """HIP translation unit for one element type and one tiling."""
     elt, esize = {"f32": ("float", 4), "f16": ("_Float16", 2)}[dtype]
     vec = 16 // esize                       # elements per 16-byte vector
@@ -81,7 +102,7 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2)):
 
     # workgroup -> macro tile, row-major over the grid of macro tiles
     nBi, nBj = size("nBi"), size("nBj")
-    Bi_e, Bj_e = OrderBy(Row(nBi, nBj)).TileBy([nBi, nBj]).inv(wg)
+    Bi_e, Bj_e = tile_order(order, nBi, nBj, wg)
     # lane -> vector of the macro tile, phase 1: SC/vec vectors per row
     v1 = OrderBy(Row(SR, SC // vec)).TileBy([SR, SC // vec]).inv(it * THREADS + t)
     v1 = [tidy(x, {t: (0, THREADS), it: (0, P1)}) for x in v1]
@@ -94,7 +115,7 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2)):
     cols_per_word = 4 // esize
     params = dict(
         banner=BANNER, elt=elt, esize=esize, SR=SR, SC=SC, KD=KD, THREADS=THREADS, P1=P1, P2=P2,
-        kernel=f"lego_transpose_{dtype}_{SR}x{SC}",
+        kernel=f"lego_transpose_{dtype}_{SR}x{SC}{suffix}",
         src_layout=f"OrderBy(Row(R, C)).TileBy([R/{SR}, C/{SC}], [{MR}, {MC}], [{TR}, {TC}])",
         dst_layout=f"OrderBy(Col(R, C)).TileBy([R/{SR}, C/{SC}], [{MR}, {MC}], [{TR}, {TC}])",
         lds_layout=f"OrderBy(GenP(({KD}, {SR}), xor-rotated rows)).TileBy([{KD}, {SR}])",
@@ -110,5 +131,5 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2)):
         grid=f"static_cast<unsigned>(rows / {SR}) * static_cast<unsigned>(cols / {SC})",
     )
     text = template("transpose.hip.j2").render(**params)
-    return Emitted(f"transpose_{dtype}.hip", text, [params["kernel"] + "_launch"]), dict(
+    return Emitted(f"transpose_{dtype}{suffix}.hip", text, [params["kernel"] + "_launch"]), dict(
         SR=SR, SC=SC, kernel=params["kernel"])

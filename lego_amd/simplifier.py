@@ -204,6 +204,18 @@ class RangeProver:
                 lo = floor(lo) if lo.is_number else (Integer(0) if self.sign_nonneg(lo) else None)
             if hi is not None and hi.is_number:
                 hi = floor(hi)
+            elif hi is not None:
+                # floor((q*d + r)/d) = q + floor(r/d): with r = -1 and d >= 1 that is q - 1,
+                # the usual "largest digit" bound of a flat index divided by a stride
+                num, den = sp.together(hi).as_numer_denom()
+                if not den.is_number and self.sign_positive(den):
+                    quot, rest = [], []
+                    for term in Add.make_args(sp.expand(num)):
+                        q = sp.cancel(term / den)
+                        (quot if q.is_integer else rest).append(q if q.is_integer else term)
+                    r = Add(*rest)
+                    if quot and r.is_number and r < 0 and self.sign_nonneg(den + r):
+                        hi = Add(*quot) - 1
             return (lo, hi)
         if isinstance(e, Mod):
             x, d = e.args

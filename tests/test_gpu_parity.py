@@ -24,8 +24,9 @@ def _gen(seed):
 # ---- transpose: bit exact ---------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype,rows,cols", [
-    (torch.float32, 64, 64), (torch.float32, 128, 320), (torch.float32, 1024, 512),
-    (torch.float16, 64, 64), (torch.float16, 192, 128), (torch.float16, 512, 1024),
+    (torch.float32, 64, 64), (torch.float32, 128, 320), (torch.float32, 1024, 512), (torch.float32, 32, 256),
+    (torch.float32, 96, 768), (torch.float16, 64, 64), (torch.float16, 192, 128), (torch.float16, 512, 1024),
+    (torch.float16, 64, 256), (torch.float16, 320, 768),
 ])
 def test_transpose_matches_oracle(ops, dtype, rows, cols):
     print(f"transpose {dtype} {rows}x{cols}", flush=True)
@@ -56,6 +57,8 @@ def test_transpose_rejects_bad_shapes(ops):
     from lego_amd.runtime import LegoHipError
     with pytest.raises(LegoHipError):
         ops.transpose(torch.zeros(100, 64, device="cuda"))
+    with pytest.raises(LegoHipError):
+        ops.transpose(torch.zeros(32, 64, device="cuda"))     # 32 rows need the 32x256 tiling
     with pytest.raises(ValueError):
         ops.transpose(torch.zeros(64, 64, device="cuda").t())
 
