@@ -20,37 +20,85 @@ from __future__ import annotations
 
 import sympy as sp
 
-from ..lego import BitXor, Col, GenP, OrderBy, Row
+from ..lego import BitXor, Col, GenP, OrderBy, Row  # noqa: F401
 from .common import BANNER, Emitted, code, idx, size, template, tidy
 
 THREADS = 256
 
 
-def staging_key(k, sr, esize):
-    """XOR key of word-column ``k`` (a multiple of 4, so 16-byte row groups stay whole).
+def lane_block(esize):
+    """Rows x vectors that the 64 lanes of one wave instruction cover in phase 1.
 
-    fp32: sixteen lanes of a wave write word-columns ``4*cv + e`` of four consecutive rows;
-    rotating the row digit by ``4*(k//4)`` sends them to 64 different banks, and the
-    sixteen 16-byte reads of one column in phase 2 cover all 64 banks once.
-    fp16: eight lanes cover one row, eight rows per instruction; ``8*(k//4)`` separates the
-    lanes of a row and ``4*(k%2)`` separates the two word-columns that share a 16-lane
-    read group in phase 2.
+    A lane scatters the four words of its vector into four word-columns at the same row
+    digit, so the lanes of one instruction must differ in the low bits of the row (which
+    stay below the XOR key) and in the vector index (which the key spreads over the
+    remaining bank bits): 4 x 16 for fp32, 8 x 8 for fp16 (whose phase 2 reads eight rows).
     """
-    if esize == 4:
-        return ((k // 4) % (sr // 4)) * 4
-    return ((k // 4) % (sr // 8)) * 8 + (k % 2) * 4
+    return (4, 16) if esize == 4 else (8, 8)
+
+
+def pack_factor(sr):
+    """Word-columns packed into one LDS row so that a row spans all 64 banks."""
+    return max(1, 64 // sr)
+
+
+def staging_key(k, sr, esize):
+    """XOR key of word-column ``k``; a multiple of 4, so 16-byte row groups stay whole.
+
+    ``LR*((k//4) % LC)`` sends the ``LC`` vectors of a phase-1 instruction to different bank
+    groups above the ``LR`` row bits; for fp16 ``4*(k%2)`` additionally separates the two
+    word-columns that share a 16-lane group of 16-byte reads in phase 2.  With a packed row
+    (``sr < 64``) the key only depends on ``k // pack_factor``, which keeps the map a
+    bijection of the row.
+    """
+    lr, lc = lane_block(esize)
+    key = ((k // 4) % lc) * lr
+    return key if esize == 4 else _xor(key, (k % 2) * 4)
+
+
+def _xor(a, b):
+    if isinstance(a, sp.Expr) or isinstance(b, sp.Expr):
+        return BitXor(sp.sympify(a), sp.sympify(b))
+    return a ^ b
+
+
+def staging_word(k, r, sr, esize):
+    """Word address of (word-column ``k``, row ``r``) in the staging tile."""
+    p = pack_factor(sr)
+    return (k // p) * (p * sr) + _xor((k % p) * sr + r, staging_key(k, sr, esize))
 
 
 def staging_layout(kd, sr, esize):
-    def forward(kr):
-        k, r = kr
-        return k * sr + BitXor(sp.sympify(r), sp.sympify(staging_key(k, sr, esize)))
+    """The staging tile as a LEGO layout: ``OrderBy(GenP((kd, sr), xor-rotated rows)).TileBy([kd, sr])``."""
+    p = pack_factor(sr)
 
     def backward(flat):
-        k, p = flat // sr, flat % sr
-        return (k, BitXor(sp.sympify(p), sp.sympify(staging_key(k, sr, esize))))
+        j, pos = flat // (p * sr), flat % (p * sr)
+        raw = _xor(pos, staging_key(j * p, sr, esize))   # the key is the same for every k of row j
+        return (j * p + raw // sr, raw % sr)
 
-    return OrderBy(GenP((kd, sr), forward, backward)).TileBy([kd, sr])
+    return OrderBy(GenP((kd, sr), lambda kr: staging_word(kr[0], kr[1], sr, esize), backward)).TileBy([kd, sr])
+
+
+def phase1_vector(sr, w, esize, it, t):
+    """``(row, vector)`` that lane ``t`` of a 256-lane workgroup loads in step ``it`` of phase 1.
+
+    The vectors of the macro tile form an ``[sr, w]`` box tiled by the lane block; a wave
+    instruction covers one block and the four waves of a step take adjacent column blocks, so
+    a step reads ``LR`` row segments of up to ``4*LC`` contiguous vectors.  Works on ints (the
+    bank-arithmetic test) and on symbols (the generator).
+    """
+    lr, lc = lane_block(esize)
+    assert sr % lr == 0 and w % lc == 0
+    symbolic = isinstance(it, sp.Expr) or isinstance(t, sp.Expr)
+    inv = (lambda lay, x: lay.inv(x)) if symbolic else (lambda lay, x: lay.inv_raw(x))
+    blocks = OrderBy(Row(sr // lr, w // lc)).TileBy([sr // lr, w // lc])
+    lanes = OrderBy(Row(lr, lc)).TileBy([lr, lc])
+    vectors = OrderBy(Row(sr, w)).TileBy([sr // lr, w // lc], [lr, lc])
+    rb, cb = inv(blocks, it * (THREADS // 64) + t // 64)
+    dr, cvl = inv(lanes, t % 64)
+    flat = vectors[rb, cb, dr, cvl] if symbolic else vectors.apply(rb, cb, dr, cvl)
+    return inv(OrderBy(Row(sr, w)).TileBy([sr, w]), flat)
 
 
 def tile_order(order, n_bi, n_bj, wg):
@@ -103,9 +151,9 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix=""):
     # workgroup -> macro tile, row-major over the grid of macro tiles
     nBi, nBj = size("nBi"), size("nBj")
     Bi_e, Bj_e = tile_order(order, nBi, nBj, wg)
-    # lane -> vector of the macro tile, phase 1: SC/vec vectors per row
-    v1 = OrderBy(Row(SR, SC // vec)).TileBy([SR, SC // vec]).inv(it * THREADS + t)
-    v1 = [tidy(x, {t: (0, THREADS), it: (0, P1)}) for x in v1]
+    # lane -> vector of the macro tile, phase 1
+    W = SC // vec
+    v1 = [tidy(x, {t: (0, THREADS), it: (0, P1)}) for x in phase1_vector(SR, W, esize, it, t)]
     # lane -> (word-column, row group), phase 2
     v2 = OrderBy(Row(KD, SR // rows_per_read)).TileBy([KD, SR // rows_per_read]).inv(it * THREADS + t)
     v2 = [tidy(x, {t: (0, THREADS), it: (0, P2)}) for x in v2]
