@@ -30,11 +30,11 @@ def lane_block(esize):
     """Rows x vectors that the 64 lanes of one wave instruction cover in phase 1.
 
     A lane scatters the four words of its vector into four word-columns at the same row
-    digit, so the lanes of one instruction must differ in the low bits of the row (which
-    stay below the XOR key) and in the vector index (which the key spreads over the
-    remaining bank bits): 4 x 16 for fp32, 8 x 8 for fp16 (whose phase 2 reads eight rows).
+    digit.  The LDS serves 4-byte accesses 32 lanes at a time over 32 banks, so the 32 lanes
+    of a pass must differ in ``address % 32``: four rows (bits 0-1, below the XOR key) times
+    eight vectors (spread by the key over bits 2-4); the other four rows form the second pass.
     """
-    return (4, 16) if esize == 4 else (8, 8)
+    return (8, 8)
 
 
 def pack_factor(sr):
@@ -45,14 +45,14 @@ def pack_factor(sr):
 def staging_key(k, sr, esize):
     """XOR key of word-column ``k``; a multiple of 4, so 16-byte row groups stay whole.
 
-    ``LR*((k//4) % LC)`` sends the ``LC`` vectors of a phase-1 instruction to different bank
-    groups above the ``LR`` row bits; for fp16 ``4*(k%2)`` additionally separates the two
+    ``4*((k//4) % 8)`` sends the eight vectors of a phase-1 pass to different groups of four
+    banks (the four rows of the pass fill a group); for fp16 ``4*(k%2)`` additionally separates the two
     word-columns that share a 16-lane group of 16-byte reads in phase 2.  With a packed row
     (``sr < 64``) the key only depends on ``k // pack_factor``, which keeps the map a
     bijection of the row.
     """
     lr, lc = lane_block(esize)
-    key = ((k // 4) % lc) * lr
+    key = ((k // 4) % lc) * 4
     return key if esize == 4 else _xor(key, (k % 2) * 4)
 
 

@@ -1,9 +1,10 @@
 """Bank arithmetic of the XOR-rotated LDS layouts (CPU only).
 
-LDS model used here: 64 banks of 4 bytes.  A wave's 4-byte accesses are served together
-(64 lanes, one bank each); 8-byte accesses in two groups of 32 lanes; 16-byte accesses in
-four groups of 16 lanes.  Within a group no two lanes may touch the same bank at different
-addresses.  On the GPU the same layouts measure SQ_LDS_BANK_CONFLICT = 0.
+LDS model, fitted to SQ_LDS_BANK_CONFLICT measurements of single-wave access patterns on
+gfx950: 4-byte accesses are served 32 lanes at a time over 32 banks (``address % 32``);
+8-byte accesses 32 lanes at a time and 16-byte reads 16 lanes at a time over 64 banks;
+16-byte writes 8 lanes at a time.  Within a pass no two lanes may touch the same bank at
+different addresses.  The GEMM layouts measure SQ_LDS_BANK_CONFLICT = 0 on the GPU.
 """
 import itertools
 
@@ -13,19 +14,18 @@ import pytest
 from lego_amd.kernels import gemm, transpose
 from oracle import lego_index as li
 
-BANKS = 64
 
-
-def conflicts(word_addrs, words_per_lane):
-    """Worst number of distinct addresses per bank within a service group (1 = conflict free)."""
-    lanes_per_group = {1: 64, 2: 32, 4: 16}[words_per_lane]
+def conflicts(word_addrs, words_per_lane, write=False):
+    """Worst number of distinct addresses per bank within a pass (1 = conflict free)."""
+    lanes_per_pass = {1: 32, 2: 32, 4: 8 if write else 16}[words_per_lane]
+    banks = 32 if words_per_lane == 1 else 64
     worst = 1
-    for g in range(0, 64, lanes_per_group):
+    for g in range(0, 64, lanes_per_pass):
         per_bank = {}
-        for lane in range(g, g + lanes_per_group):
+        for lane in range(g, g + lanes_per_pass):
             for w in range(words_per_lane):
                 a = int(word_addrs[lane]) + w
-                per_bank.setdefault(a % BANKS, set()).add(a)
+                per_bank.setdefault(a % banks, set()).add(a)
         worst = max(worst, max(len(s) for s in per_bank.values()))
     return worst
 
@@ -87,8 +87,8 @@ def test_gemm_lds_layouts_are_bijective_and_conflict_free():
     # global->LDS stores: lane t holds chunk (t % 8) of row (t / 8) of A, chunk (t % 32) of k-row (t / 32) of B
     for wave in range(4):
         lanes = [wave * 64 + l for l in range(64)]
-        assert conflicts([4 * ta[t // 8, t % 8] for t in lanes], 4) == 1
-        assert conflicts([tb[t // 32, 8 * (t % 32)] // 2 for t in lanes], 4) == 1
+        assert conflicts([4 * ta[t // 8, t % 8] for t in lanes], 4, write=True) == 1
+        assert conflicts([tb[t // 32, 8 * (t % 32)] // 2 for t in lanes], 4, write=True) == 1
     # A fragments: lane l reads chunk (2*ks + l/32) of row (l % 32) -> ds_read_b128
     for ks in range(4):
         assert conflicts([4 * ta[l % 32, 2 * ks + l // 32] for l in range(64)], 4) == 1
@@ -102,7 +102,7 @@ def test_gemm_lds_layouts_are_bijective_and_conflict_free():
 
 
 def test_oracle_xor_swizzle_matches_product_family():
-    blk = li.xor_swizzle(16, 64, unit=4, every=4, span=16)
+    blk = li.xor_swizzle(16, 64, unit=4, every=4, span=16)   # fp32 key of a 64-row tile, 16 vectors
     seen = set()
     for r, c in itertools.product(range(16), range(64)):
         p = blk.apply((r, c))
