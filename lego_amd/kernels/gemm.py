@@ -64,6 +64,24 @@ def lds_b_layout(bk, bn):
     return OrderBy(GenP((bk, bn), forward, backward)).TileBy([bk, bn])
 
 
+def lds_c_layout(rows, cols):
+    """A wave's block of C as fp16 in 8-byte chunks: ``row*(cols/4) + (chunk ^ (row % 32))``.
+
+    The accumulator layout makes 32 lanes store the same chunk of 32 consecutive rows; the
+    rotation spreads them over 32 different chunks of the 256-byte bank window."""
+    chunks = cols // 4
+
+    def forward(rc):
+        row, ch = rc
+        return row * chunks + BitXor(sp.sympify(ch), sp.sympify(row % 32))
+
+    def backward(flat):
+        row, p = flat // chunks, flat % chunks
+        return (row, BitXor(sp.sympify(p), sp.sympify(row % 32)))
+
+    return OrderBy(GenP((rows, chunks), forward, backward)).TileBy([rows, chunks])
+
+
 def launch_order(num_pid_m, num_pid_n, group_m, pid):
     """``(pid_m, pid_n)`` of the grouped launch order (matmul_sympy.py:57-65)."""
     lay = OrderBy(Col(sp.Max(num_pid_m // group_m, 1), 1),
@@ -103,11 +121,6 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
     As_L = lds_a_layout(bm, bk // 8)
     Bs_L = lds_b_layout(bk, bn)
 
-    lane_rng = {t: (0, THREADS), it: (0, max(A_ITERS, B_ITERS))}
-    a_row, a_ch = (tidy(e, lane_rng) for e in
-                   OrderBy(Row(bm, bk // 8)).TileBy([bm, bk // 8]).inv(it * THREADS + t))
-    b_kr, b_ch = (tidy(e, lane_rng) for e in
-                  OrderBy(Row(bk, bn // 8)).TileBy([bk, bn // 8]).inv(it * THREADS + t))
     wm_e, wn_e = OrderBy(Row(WAVES_M, WAVES_N)).TileBy([WAVES_M, WAVES_N]).inv(wave)
 
     rng = {row: (0, bm), ch: (0, bk // 8), kr: (0, bk), i: (0, TM), j: (0, TN), r: (0, 16),
@@ -118,32 +131,51 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
     def chunk_walk(expr, n_iters):
         """``expr`` (a function of the lane ``t`` and the chunk counter ``it``) as
         ``expr(it=0) + it*step`` with a lane-independent ``step``; raises if it is not."""
-        at = [tidy(sp.sympify(expr).subs(it, v), {t: (0, THREADS)}) for v in range(n_iters)]
+        lane_s, rng_l = idx("lane"), {idx("lane"): (0, 64), wave: (0, WAVES_M * WAVES_N)}
+        at = [tidy(sp.sympify(expr).subs(it, v), rng_l) for v in range(n_iters)]
         step = sp.simplify(at[1] - at[0]) if n_iters > 1 else sp.Integer(0)
-        if t in step.free_symbols:
-            raise ValueError(f"chunk stride depends on the lane: {step}")
-        for v in range(n_iters):   # exhaustive over lanes: the walk really is affine
-            for lane in range(THREADS):
-                if (at[v] - at[0] - v * step).subs(t, lane) != 0:
-                    raise ValueError("chunk offsets are not affine in the chunk counter")
+        if step.free_symbols & {lane_s, wave}:
+            # not visibly uniform: decide by exhaustive evaluation below
+            step = sp.simplify((at[1] - at[0]).subs({lane_s: 0, wave: 0}))
+        sizes = {s_: 8192 + 256 * n_ for n_, s_ in enumerate(sorted(step.free_symbols | at[0].free_symbols
+                                                                   - {lane_s, wave}, key=str))}
+        for v in range(n_iters):   # exhaustive over lanes and waves: the walk really is affine
+            diff = sp.lambdify([lane_s, wave], (at[v] - at[0] - v * step).subs(sizes), "math")
+            for w_ in range(WAVES_M * WAVES_N):
+                for l_ in range(64):
+                    if diff(l_, w_) != 0:
+                        raise ValueError("chunk offsets are not affine in the instruction counter")
         return at[0], step
+
+    Cs_L = lds_c_layout(WM, WN)
+    cp = idx("cp")
+    rng.update({cr: (0, WM), cp: (0, WN // 8)})
+    lane_o = idx("lane")
+    c_out = [tidy(e, {lane_o: (0, 64), it: (0, WM * WN // 8 // 64)}) for e in
+             OrderBy(Row(WM, WN // 8)).TileBy([WM, WN // 8]).inv(it * 64 + lane_o)]
 
     frag_row = wm * WM + i * 32 + l32
     frag_k = [ks * 16 + (lgrp // 2) * 8 + h * 4 + l16 // 4 for h in (0, 1)]
     frag_n = wn * WN + j * 32 + (lgrp % 2) * 16 + 4 * (l16 % 4)
     pm_e, pn_e = launch_order(npm, npn, group_m, pid)
 
+    # memory->LDS: instruction `it` of wave `wave` fills slots (it*WAVES + wave)*64 + lane; the chunk
+    # that lives in a slot is the inverse of the LDS layout
+    WAVES = WAVES_M * WAVES_N
+    lane_s = idx("lane")
+    slot = (it * WAVES + wave) * 64 + lane_s
+    slot_rng = {lane_s: (0, 64), wave: (0, WAVES), it: (0, max(A_ITERS, B_ITERS))}
+    a_row, a_ch = (tidy(e, slot_rng) for e in As_L.inv(slot))
+    b_kr, b_n = (tidy(e, slot_rng) for e in Bs_L.inv(8 * slot))
+    b_ch = tidy(b_n / 8, slot_rng)
     sub_a = {row: a_row, ch: a_ch}
     sub_b = {kr: b_kr, ch: b_ch}
     a_full = tidy(A_L[pid_m, k, row, ch * 8], rng)     # the reference's a_ptrs expression
     b_full = tidy(B_L[k, pid_n, kr, ch * 8], rng)     # and its b_ptrs expression
     a_src0, a_src_step = chunk_walk(a_full.subs({pid_m: 0, k: 0}).subs(sub_a), A_ITERS)
     b_src0, b_src_step = chunk_walk(b_full.subs({pid_n: 0, k: 0}).subs(sub_b), B_ITERS)
-    a_dst0, a_dst_step = chunk_walk(tidy(8 * As_L[row, ch], rng).subs(sub_a), A_ITERS)
-    b_dst0, b_dst_step = chunk_walk(tidy(Bs_L[kr, ch * 8], rng).subs(sub_b), B_ITERS)
     chunk_params = dict(a_src0=code(a_src0), a_src_step=code(a_src_step), b_src0=code(b_src0),
-                        b_src_step=code(b_src_step), a_dst0=code(a_dst0), a_dst_step=code(a_dst_step),
-                        b_dst0=code(b_dst0), b_dst_step=code(b_dst_step))
+                        b_src_step=code(b_src_step), WAVES=WAVES)
 
     params = dict(
         banner=BANNER, BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
@@ -155,21 +187,22 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
         b_layout=f"OrderBy(Row(K,N)).TileBy([K/{bk},N/{bn}],[{bk},{bn}])",
         c_layout=f"OrderBy(Row(M,N)).TileBy([M/{bm},N/{bn}],[{bm},{bn}])",
         wm=code(wm_e), wn=code(wn_e),
-        a_row=code(a_row), a_ch=code(a_ch), b_kr=code(b_kr), b_ch=code(b_ch),
         # offset of a chunk = tile base (uniform) + position inside k-tile 0 (per lane) + k * step
         **chunk_params,
         a_goff_base=code(a_full.subs({k: 0, row: 0, ch: 0})),
         b_goff_base=code(b_full.subs({k: 0, kr: 0, ch: 0})),
         a_kstep=code(sp.simplify(a_full.subs(k, k + 1) - a_full)),
         b_kstep=code(sp.simplify(b_full.subs(k, k + 1) - b_full)),
-        a_loff=code(tidy(8 * As_L[row, ch], rng)),
-        b_loff=code(tidy(Bs_L[kr, ch * 8], rng)),
         a_frag=code(tidy(8 * As_L[frag_row, ks * 2 + lhi], rng)),
         b_frag0=code(tidy(Bs_L[frag_k[0], frag_n], rng)),
         b_frag1=code(tidy(Bs_L[frag_k[1], frag_n], rng)),
-        c_row=code(wm * WM + i * 32 + l32),
-        c_col=code(wn * WN + j * 32 + q * 8 + lhi * 4),
-        c_goff=code(tidy(C_L[pid_m, pid_n, cr, cc], rng)),
+        # accumulator -> staging: row i*32 + l32, 8-byte chunk (j*32 + q*8 + lhi*4)/4 of the wave's block
+        c_stage_store=code(tidy(4 * Cs_L[i * 32 + l32, j * 8 + q * 2 + lhi], rng)),
+        # staging -> memory: lane reads the pair of chunks (2p, 2p+1) of row cr; the XOR keeps a
+        # pair together and swaps its halves on odd rows
+        c_out_row=code(c_out[0]), c_out_pair=code(c_out[1]),
+        c_stage_load=code(tidy(4 * Cs_L[cr, 2 * cp], rng) - 4 * (cr % 2)),
+        c_goff=code(tidy(C_L[pid_m, pid_n, wm * WM + cr, wn * WN + 8 * cp], rng)),
         xcd_pid=code(tidy(xcd_remap(per_xcd, wg), {wg: (0, per_xcd * XCDS)})),
         pid_m=code(pm_e), pid_n=code(pn_e),
     )

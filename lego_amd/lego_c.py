@@ -10,7 +10,24 @@ from sympy.printing.precedence import precedence
 from .lego import *  # noqa: F401,F403
 
 
-class LEGOCCodePrinter(C99CodePrinter):
+class NegativeProductMixin:
+    """Prints ``-c*x`` as ``-`` followed by the product ``c*x``.
+
+    sympy's code printers compute the parenthesisation level of a product before they strip
+    its minus sign; a negative product therefore prints its factors at the level of a sum and
+    ``x - 4*Mod(r, 2)`` comes out as ``x - 4*r % 2``, which C and Python read as
+    ``x - (4*r) % 2``.  Printing the positive product on its own keeps the parentheses."""
+
+    def _print_Mul(self, expr):
+        coeff, _ = expr.as_coeff_Mul()
+        if coeff.is_negative:
+            positive = -expr
+            text = self._print(positive)
+            return "-(" + text + ")" if isinstance(positive, sp.Mod) else "-" + text
+        return super()._print_Mul(expr)
+
+
+class LEGOCCodePrinter(NegativeProductMixin, C99CodePrinter):
     def __init__(self, settings=None, **kwargs):
         merged = dict(settings or {})
         merged.update(kwargs)

@@ -7,9 +7,10 @@ and a ``TritonRange`` becomes a broadcast slice of its index vector.
 from sympy.printing.pycode import PythonCodePrinter
 
 from .lego import *  # noqa: F401,F403
+from .lego_c import NegativeProductMixin
 
 
-class LEGOPythonCodePrinter(PythonCodePrinter):
+class LEGOPythonCodePrinter(NegativeProductMixin, PythonCodePrinter):
     """``LEGOPythonCodePrinter(allow_unknown_functions=True, do_broadcast=True)``."""
 
     def __init__(self, settings=None, **kwargs):

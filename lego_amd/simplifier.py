@@ -25,6 +25,10 @@ from __future__ import annotations
 import sympy as sp
 from sympy import Add, Integer, Mod, Mul, Pow, Rational, floor
 
+from . import sympy_compat
+
+sympy_compat.install()
+
 __all__ = ["simplify_ops", "RangeProver", "BitXor"]
 
 

@@ -77,3 +77,24 @@ def test_builder_module_compiles_for_gfx950(tmp_path):
     res = subprocess.run([hipcc_path(), *HIPCC_FLAGS, "--cuda-device-only", "-c", str(src), "-o", str(tmp_path / "k.o")],
                          capture_output=True, text=True)
     assert res.returncode == 0, res.stderr
+
+
+def test_negative_products_keep_their_parentheses():
+    """sympy prints x - 4*Mod(r, 2) as 'x - 4*r % 2'; C and Python read that as x - (4*r) % 2."""
+    from lego_amd.lego_python import LEGOPythonCodePrinter
+    r, x = sp.symbols("r x", integer=True, nonnegative=True)
+    for pr in (LEGOHipCodePrinter(), LEGOPythonCodePrinter()):
+        for expr in (x - 4 * sp.Mod(r, 2), x - sp.Mod(r, 2), 7 - x * sp.Mod(r, 3), -sp.Mod(r, 2) + 9):
+            text = pr.doprint(expr).replace("/", "//")
+            for rv in range(6):
+                for xv in range(4):
+                    assert eval(text, {}, {"r": rv, "x": xv}) == expr.subs({r: rv, x: xv}), (expr, text)
+
+
+def test_sympy_mod_product_defect_is_guarded():
+    """Mod(8*Mod(y, 2048), 256) must stay a function that equals (8*(y % 2048)) % 256."""
+    y = sp.Symbol("y", integer=True, nonnegative=True)
+    for c, n, q in [(8, 2048, 256), (3, 5, 7), (6, 10, 4), (4, 3, 8), (12, 7, 18)]:
+        e = sp.Mod(c * sp.Mod(y, n), q)
+        for v in range(0, 80, 3):
+            assert int(e.subs(y, v)) == (c * (v % n)) % q
