@@ -105,6 +105,7 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
     A_ITERS = bm * bk // 8 // THREADS
     B_ITERS = bk * bn // 8 // THREADS
     assert bm * bk // 8 % THREADS == 0 and bk * bn // 8 % THREADS == 0 and bk % 16 == 0
+    assert WN >= 128, "the epilogue's staging rotation needs 32 eight-byte chunks per row"
 
     M, N, K = size("M"), size("N"), size("K")
     npm, npn, per_xcd, group_m = size("num_pid_m"), size("num_pid_n"), size("wg_per_xcd"), size("GM")
