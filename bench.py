@@ -103,10 +103,13 @@ def main():
     gbs2 = bytes2 / ms2 / 1e6
     copy_ms = timed(lambda: y2.copy_(x2))
     copy_gbs = bytes2 / copy_ms / 1e6
+    copy16_ms = timed(lambda: runtime.call("lego_hip_copy16", p(x2), p(y2), ctypes.c_ulonglong(bytes2 // 2), stream))
     kernels["c2_transpose_f16_16384"] = dict(ms=ms2, gbs=gbs2, frac_hbm=gbs2 / HBM_PEAK_GBS,
                                              bytes=bytes2, parity="bit-exact")
     kernels["device_copy_512MiB"] = dict(ms=copy_ms, gbs=copy_gbs, frac_hbm=copy_gbs / HBM_PEAK_GBS,
                                          note="torch copy_ of the same buffers: achievable ceiling")
+    kernels["device_copy16_512MiB"] = dict(ms=copy16_ms, gbs=bytes2 / copy16_ms / 1e6,
+                                           note="plain 16-byte-per-lane copy kernel of this library (counter calibration)")
 
     # ---- C1: fp32 4096^2 transpose ---------------------------------------------------------
     if want("c1"):

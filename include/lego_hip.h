@@ -29,16 +29,20 @@ int lego_hip_abi_version(void);
 int lego_hip_transpose_f32(const void* in, void* out, int rows, int cols, void* stream);
 int lego_hip_transpose_f16(const void* in, void* out, int rows, int cols, void* stream);
 
-/* y = softmax(x) over the last dimension of an M x N fp16 matrix, fp32 arithmetic.
- * Replaces softmax(x) (reference: triton_generated/softmax/softmax.py:97-160).
- * N must be a multiple of 8 and at most 16384. */
+/* y = softmax(x) over the last dimension of an M x N matrix (fp16 or fp32 in/out), fp32
+ * arithmetic.  Replaces softmax(x) (reference: triton_generated/softmax/softmax.py:97-160; the
+ * reference's own test is a ragged fp32 1823 x 781 matrix, softmax.py:237-241).
+ * Any N up to 16384; rows whose length is a multiple of 16 bytes take the 16-byte-access path. */
 int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream);
+int lego_hip_softmax_f32(const void* x, void* y, int M, int N, void* stream);
 
-/* LayerNorm forward over the last dimension of an M x N fp16 matrix; w, b are fp16 [N];
- * mean, rstd are fp32 [M] outputs.  Replaces LEGOLayerNorm.forward / lego_layer_norm
- * (reference: triton_generated/layernorm/layernorm.py:279-307).
- * N must be a multiple of 8 and at most 16384. */
+/* LayerNorm forward over the last dimension of an M x N matrix; x, y, w, b share one element
+ * type (fp16 or fp32), w and b have N elements; mean, rstd are fp32 [M] outputs.  Replaces
+ * LEGOLayerNorm.forward / lego_layer_norm (reference:
+ * triton_generated/layernorm/layernorm.py:279-307).  Any N up to 16384. */
 int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void* b,
+                               float* mean, float* rstd, int M, int N, float eps, void* stream);
+int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void* b,
                                float* mean, float* rstd, int M, int N, float eps, void* stream);
 
 /* C = A * B, A is M x K, B is K x N, C is M x N, fp16 with fp32 accumulation.
@@ -57,11 +61,16 @@ int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* 
                               const int* sizes3, int groups, void* stream);
 
 /* Tuning entry points: as above, with the launch shape chosen by the caller
- * (waves_per_row in {1, 2, 4}).  Used by the benchmark to compare variants. */
+ * (waves_per_row in {1, 2, 4}; N a multiple of 8).  Used by the benchmark to compare variants. */
 int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per_row, void* stream);
 int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const void* b,
                                    float* mean, float* rstd, int M, int N, float eps,
                                    int waves_per_row, void* stream);
+
+/* Measurement aid: out[0..bytes) = in[0..bytes), 16 bytes per lane per access, bytes % 16 == 0.
+ * No counterpart in the reference.  bench.py uses it as the same-run copy ceiling and the
+ * profiles use it to calibrate the FETCH_SIZE / WRITE_SIZE counters at this access width. */
+int lego_hip_copy16(const void* in, void* out, unsigned long long bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -33,7 +33,10 @@ TRANSPOSE = {
     "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag"),
             dict(dtype="f16", tile=(64, 64), group=(1, 1), order="diag")],
 }
-ROWWISE_WAVES = (1, 2, 4)
+# (element type, vectorised, waves per row): 16-byte accesses need N % (16/size) == 0; the
+# element-per-access kernels ("s") take any N
+ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f32", True, 1), ("f32", True, 4),
+           ("f16", False, 4), ("f32", False, 4)]
 ROWWISE_DEFAULT_WAVES = 4
 ROWWISE_MAX_N = 16384
 GEMM = dict(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8)
@@ -49,7 +52,7 @@ def generate():
             unit.filename = f"transpose_{dtype}_{meta['SR']}x{meta['SC']}.hip"
             units.append(unit)
             tmeta.setdefault(dtype, []).append(meta)
-    units += [rowwise.emit(w) for w in ROWWISE_WAVES]
+    units += [rowwise.emit(w, dtype, vec) for dtype, vec, w in ROWWISE]
     g, mg = gemm.emit(**GEMM)
     units.append(g)
 
@@ -64,9 +67,10 @@ def generate():
             h.append(f"  if (rows % {m['SR']} == 0 && cols % {m['SC']} == 0) "
                      f"return {m['kernel']}_launch(in, out, rows, cols, stream);")
         h += ["  return hipErrorInvalidValue;", "}", ""]
-    for w in ROWWISE_WAVES:
-        h += [f"hipError_t lego_softmax_f16_w{w}_launch(const void*, void*, int, int, hipStream_t);",
-              f"hipError_t lego_layernorm_fwd_f16_w{w}_launch(const void*, void*, const void*, const void*, "
+    for dtype, vec, w in ROWWISE:
+        tag = dtype if vec else dtype + "s"
+        h += [f"hipError_t lego_softmax_{tag}_w{w}_launch(const void*, void*, int, int, hipStream_t);",
+              f"hipError_t lego_layernorm_fwd_{tag}_w{w}_launch(const void*, void*, const void*, const void*, "
               "float*, float*, int, int, float, hipStream_t);"]
     h += [f"#define LEGO_ROWWISE_MAX_N {ROWWISE_MAX_N}",
           "// waves per row: one wave keeps short rows free of barriers, four waves keep the",

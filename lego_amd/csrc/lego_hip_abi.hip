@@ -19,6 +19,13 @@ inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 inline int ok_or(hipError_t e) { return static_cast<int>(e); }
 constexpr int kInvalid = static_cast<int>(hipErrorInvalidValue);
 
+// plain grid-stride copy, one 16-byte vector per lane per step
+__global__ void __launch_bounds__(256) lego_copy16_kernel(const uint4* __restrict__ in, uint4* __restrict__ out, size_t n)
+{
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = in[i];
+}
+
 }  // namespace
 
 extern "C" {
@@ -53,7 +60,17 @@ int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per
 
 int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream)
 {
+  if (!usable(x) || !usable(y) || M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N) return kInvalid;
+  if (N % 8) return ok_or(lego_softmax_f16s_w4_launch(x, y, M, N, as_stream(stream)));   // ragged rows
   return lego_hip_softmax_f16_wpr(x, y, M, N, lego_rowwise_default_wpr(N), stream);
+}
+
+int lego_hip_softmax_f32(const void* x, void* y, int M, int N, void* stream)
+{
+  if (!usable(x) || !usable(y) || M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N) return kInvalid;
+  if (N % 4) return ok_or(lego_softmax_f32s_w4_launch(x, y, M, N, as_stream(stream)));   // ragged rows
+  if (N <= 1024) return ok_or(lego_softmax_f32_w1_launch(x, y, M, N, as_stream(stream)));
+  return ok_or(lego_softmax_f32_w4_launch(x, y, M, N, as_stream(stream)));
 }
 
 int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const void* b,
@@ -73,7 +90,20 @@ int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const 
 int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void* b,
                                float* mean, float* rstd, int M, int N, float eps, void* stream)
 {
+  if (!usable(x) || !usable(y) || !usable(w) || !usable(b) || mean == nullptr || rstd == nullptr) return kInvalid;
+  if (M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
+  if (N % 8) return ok_or(lego_layernorm_fwd_f16s_w4_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
   return lego_hip_layernorm_fwd_f16_wpr(x, y, w, b, mean, rstd, M, N, eps, lego_rowwise_default_wpr(N), stream);
+}
+
+int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void* b,
+                               float* mean, float* rstd, int M, int N, float eps, void* stream)
+{
+  if (!usable(x) || !usable(y) || !usable(w) || !usable(b) || mean == nullptr || rstd == nullptr) return kInvalid;
+  if (M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
+  if (N % 4) return ok_or(lego_layernorm_fwd_f32s_w4_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+  if (N <= 1024) return ok_or(lego_layernorm_fwd_f32_w1_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+  return ok_or(lego_layernorm_fwd_f32_w4_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
 }
 
 int lego_hip_gemm_f16(const void* a, const void* b, void* c, int M, int N, int K, void* stream)
@@ -94,6 +124,16 @@ int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* 
     if (m <= 0 || n <= 0 || k <= 0 || m % LEGO_GEMM_BM || n % LEGO_GEMM_BN || k % LEGO_GEMM_BK) return kInvalid;
   }
   return ok_or(lego_grouped_gemm_f16_launch(a, b, c, sizes3, groups, as_stream(stream)));
+}
+
+int lego_hip_copy16(const void* in, void* out, unsigned long long bytes, void* stream)
+{
+  if (!usable(in) || !usable(out) || bytes == 0 || bytes % 16) return kInvalid;
+  const size_t n = bytes / 16;
+  const unsigned grid = static_cast<unsigned>(n / 256 < 256 * 32 ? (n + 255) / 256 : 256 * 32);
+  hipLaunchKernelGGL(lego_copy16_kernel, dim3(grid), dim3(256), 0, as_stream(stream),
+                     static_cast<const uint4*>(in), static_cast<uint4*>(out), n);
+  return ok_or(hipGetLastError());
 }
 
 }  // extern "C"

@@ -20,11 +20,18 @@ from ..lego import OrderBy, Row
 from .common import BANNER, Emitted, code, idx, size, template, tidy
 
 THREADS = 256
-VPTS = (1, 2, 4, 8, 16)
+MAX_N = 16384
+VPTS = (1, 2, 4, 8, 16, 32, 64)
 
 
-def emit(waves_per_row=1):
+def emit(waves_per_row=1, dtype="f16", vectorised=True):
+    """One translation unit: every register footprint ``V`` of one (waves per row, element type,
+    access width) combination.  ``vectorised=False`` emits the element-per-access kernels that
+    take rows of any length and alignment (the reference's own softmax test is 1823 x 781)."""
     WPR = waves_per_row
+    elt, esize = {"f16": ("_Float16", 2), "f32": ("float", 4)}[dtype]
+    EPV = 16 // esize if vectorised else 1
+    tag = dtype if vectorised else dtype + "s"
     TEAM = 64 * WPR
     RPW = THREADS // TEAM                       # rows per workgroup
     M, N, NWG = size("M"), size("N"), size("NWG")
@@ -36,22 +43,24 @@ def emit(waves_per_row=1):
     rows = OrderBy(Row(NWG, RPW)).TileBy([NWG], [RPW])
     row_e = tidy(rows[wg, team], {wg: (0, NWG), team: (0, RPW)})
     # x[row][vector][8]: vector v = it*TEAM + lane of the row, as an offset in elements
-    X = OrderBy(Row(M, N)).TileBy([M, N / 8], [1, 8])
+    X = OrderBy(Row(M, N)).TileBy([M, N / EPV], [1, EPV])
     vec_e = it * TEAM + lane
     row_base = tidy(X[row, 0, 0, 0], {row: (0, M)})
-    vec_off = tidy(X[0, v, 0, 0], {v: (0, N / 8)})
+    vec_off = tidy(X[0, v, 0, 0], {v: (0, N / EPV)})
     stat = OrderBy(Row(M)).TileBy([M])[row,]
 
     params = dict(
         banner=BANNER, WPR=WPR, TEAM=TEAM, RPW=RPW, THREADS=THREADS,
-        VPTS=[vp for vp in VPTS if vp * TEAM * 8 <= 65536],
+        # a lane keeps V*EPV fp32 values: at most 128, and no more footprints than MAX_N needs
+        VPTS=[vp for vp in VPTS if vp * EPV <= 128 and vp * TEAM * EPV <= MAX_N],
+        dtype=dtype, elt=elt, EPV=EPV, tag=tag,
         row_layout=f"OrderBy(Row(NWG, {RPW})).TileBy([NWG], [{RPW}])[wg, team]",
         lane_layout=f"OrderBy(Row({RPW}, {TEAM})).TileBy([{RPW}, {TEAM}]).inv(t); vector = it*{TEAM} + lane",
-        x_layout="OrderBy(Row(M, N)).TileBy([M, N/8], [1, 8])[row, v, 0, :]",
+        x_layout=f"OrderBy(Row(M, N)).TileBy([M, N/{EPV}], [1, {EPV}])[row, v, 0, :]",
         team=code(team_e), lane=code(lane_e), row=code(row_e),
         row_base=code(row_base).replace("row", "static_cast<size_t>(row)"),
         vec=code(vec_e), vec_off=code(vec_off), stat_off=code(stat),
     )
     text = template("rowwise.hip.j2").render(**params)
-    return Emitted(f"rowwise_w{WPR}.hip", text,
-                   [f"lego_softmax_f16_w{WPR}_launch", f"lego_layernorm_fwd_f16_w{WPR}_launch"])
+    return Emitted(f"rowwise_{tag}_w{WPR}.hip", text,
+                   [f"lego_softmax_{tag}_w{WPR}_launch", f"lego_layernorm_fwd_{tag}_w{WPR}_launch"])

@@ -21,6 +21,9 @@ SIGNATURES = {
     "lego_hip_transpose_f32": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "lego_hip_transpose_f16": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "lego_hip_softmax_f16": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+    "lego_hip_softmax_f32": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+    "lego_hip_layernorm_fwd_f32": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                                   _c_int, _c_int, _c_float, _c_void_p],
     "lego_hip_layernorm_fwd_f16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                    _c_int, _c_int, _c_float, _c_void_p],
     "lego_hip_gemm_f16": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
@@ -28,6 +31,7 @@ SIGNATURES = {
     "lego_hip_softmax_f16_wpr": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "lego_hip_layernorm_fwd_f16_wpr": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                        _c_int, _c_int, _c_float, _c_int, _c_void_p],
+    "lego_hip_copy16": [_c_void_p, _c_void_p, ctypes.c_ulonglong, _c_void_p],
 }
 
 _lib = None

@@ -84,6 +84,44 @@ def test_softmax_matches_oracle(ops, M, N, wpr):
     assert torch.allclose(got.float().sum(-1), torch.ones(M), atol=2e-2)
 
 
+def test_softmax_reference_test_shape_fp32(ops):
+    """The reference's own check (softmax.py:237-241): seed 0, x = randn(1823, 781) in fp32,
+    compared with torch.softmax at allclose's default tolerance."""
+    print("softmax fp32 1823x781", flush=True)
+    torch.manual_seed(0)
+    x = torch.randn(1823, 781)
+    got = ops.softmax(x.cuda()).cpu()
+    assert torch.allclose(got, torch.softmax(x, dim=1))
+    assert (got - ok.softmax(x)).abs().max().item() <= 1e-6
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("M,N", [(5, 1), (9, 3), (17, 781), (4, 1000), (3, 4099), (2, 16383), (6, 2048), (3, 16384)])
+def test_softmax_ragged_and_fp32(ops, dtype, M, N):
+    print(f"softmax {dtype} {M}x{N}", flush=True)
+    x = (2.0 * torch.randn(M, N, generator=_gen(2))).to(dtype)
+    want = ok.softmax(x)
+    got = ops.softmax(x.cuda()).cpu()
+    assert (got.float() - want.float()).abs().max().item() <= (TOL if dtype == torch.float16 else 1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("M,N", [(5, 1), (9, 3), (17, 781), (3, 4099), (6, 2048), (3, 16384)])
+def test_layernorm_ragged_and_fp32(ops, dtype, M, N):
+    print(f"layernorm {dtype} {M}x{N}", flush=True)
+    g = _gen(3)
+    x = (2.0 * torch.randn(M, N, generator=g)).to(dtype)
+    w = (1 + 0.1 * torch.randn(N, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(N, generator=g)).to(dtype)
+    want_y, want_mean, want_rstd = ok.layernorm_fwd(x, w, b, 1e-5)
+    y, mean, rstd = ops.layer_norm_fwd(x.cuda(), w.cuda(), b.cuda(), 1e-5)
+    tol = 2 * TOL if dtype == torch.float16 else 2e-5
+    assert (y.cpu().float() - want_y.float()).abs().max().item() <= tol
+    assert torch.allclose(mean.cpu(), want_mean, atol=1e-4, rtol=1e-4)
+    if N > 1:
+        assert torch.allclose(rstd.cpu(), want_rstd, atol=1e-4, rtol=1e-3)
+
+
 @pytest.mark.parametrize("wpr", [None, 1, 2, 4])
 @pytest.mark.parametrize("M,N", [(7, 8), (33, 520), (64, 1024), (129, 4096), (1151, 8192), (3, 16384)])
 def test_layernorm_matches_oracle(ops, M, N, wpr):
