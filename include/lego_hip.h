@@ -45,6 +45,18 @@ int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void
 int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void* b,
                                float* mean, float* rstd, int M, int N, float eps, void* stream);
 
+/* LayerNorm backward: dx (M x N fp16), dw and db (N fp16) from dy, x, w and the forward pass's
+ * mean and rstd.  Replaces LEGOLayerNorm.backward (reference:
+ * triton_generated/layernorm/layernorm.py:162-268, host side :372-405), whose lock-guarded
+ * partial buffers become one fp32 workspace the caller provides (the reference's wrapper
+ * allocates its buffers with torch as well): ask for its size first, any 16-byte aligned
+ * device buffer of at least that many bytes will do; its contents need no initialisation.
+ * N must be a multiple of 8 and at most 8192. */
+int lego_hip_layernorm_bwd_workspace_bytes(int M, int N, unsigned long long* bytes);
+int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, const float* mean,
+                               const float* rstd, void* dx, void* dw, void* db, void* workspace,
+                               unsigned long long workspace_bytes, int M, int N, void* stream);
+
 /* C = A * B, A is M x K, B is K x N, C is M x N, fp16 with fp32 accumulation.
  * Replaces matmul(a, b) (reference: triton_generated/matmul/matmul_NTA_NTB.py:129-145).
  * Like the reference kernel (no edge masks, matmul_sympy.py:196-203) the sizes must divide

@@ -14,7 +14,7 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
-from .kernels import gemm, rowwise, transpose
+from .kernels import gemm, layernorm_bwd, rowwise, transpose
 from .kernels.common import BANNER, CSRC, GENERATED
 from .lego_hip import HIPCC_FLAGS, hipcc_path
 
@@ -55,6 +55,8 @@ def generate():
     units += [rowwise.emit(w, dtype, vec) for dtype, vec, w in ROWWISE]
     g, mg = gemm.emit(**GEMM)
     units.append(g)
+    lb, mlb = layernorm_bwd.emit()
+    units.append(lb)
 
     h = [f"// {BANNER}", "#pragma once", "#include <hip/hip_runtime.h>", ""]
     for dtype, metas in tmeta.items():
@@ -76,6 +78,10 @@ def generate():
           "// waves per row: one wave keeps short rows free of barriers, four waves keep the",
           "// register footprint of long rows small enough for full occupancy",
           f"inline int lego_rowwise_default_wpr(int n) {{ return n <= 2048 ? 1 : {ROWWISE_DEFAULT_WAVES}; }}", ""]
+    h += ["unsigned lego_layernorm_bwd_groups(int M);",
+          "hipError_t lego_layernorm_bwd_f16_launch(const void*, const void*, const void*, const float*, const float*, "
+          "void*, void*, void*, float*, int, int, hipStream_t);",
+          f"#define LEGO_LAYERNORM_BWD_MAX_N {mlb['MAX_N']}", ""]
     h += ["hipError_t lego_gemm_f16_launch(const void*, const void*, void*, int, int, int, hipStream_t);",
           "hipError_t lego_grouped_gemm_f16_launch(const void* const*, const void* const*, void* const*, "
           "const int*, int, hipStream_t);",

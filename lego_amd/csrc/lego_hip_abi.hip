@@ -106,6 +106,26 @@ int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void
   return ok_or(lego_layernorm_fwd_f32_w4_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
 }
 
+int lego_hip_layernorm_bwd_workspace_bytes(int M, int N, unsigned long long* bytes)
+{
+  if (bytes == nullptr || M <= 0 || N <= 0 || N % 8 || N > LEGO_LAYERNORM_BWD_MAX_N) return kInvalid;
+  *bytes = 2ull * lego_layernorm_bwd_groups(M) * static_cast<unsigned long long>(N) * sizeof(float);
+  return 0;
+}
+
+int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, const float* mean,
+                               const float* rstd, void* dx, void* dw, void* db, void* workspace,
+                               unsigned long long workspace_bytes, int M, int N, void* stream)
+{
+  unsigned long long need = 0;
+  if (lego_hip_layernorm_bwd_workspace_bytes(M, N, &need) != 0) return kInvalid;
+  if (!usable(dy) || !usable(x) || !usable(w) || !usable(dx) || !usable(dw) || !usable(db) || !usable(workspace))
+    return kInvalid;
+  if (mean == nullptr || rstd == nullptr || workspace_bytes < need) return kInvalid;
+  return ok_or(lego_layernorm_bwd_f16_launch(dy, x, w, mean, rstd, dx, dw, db, static_cast<float*>(workspace), M, N,
+                                             as_stream(stream)));
+}
+
 int lego_hip_gemm_f16(const void* a, const void* b, void* c, int M, int N, int K, void* stream)
 {
   if (!usable(a) || !usable(b) || !usable(c)) return kInvalid;

@@ -1,0 +1,44 @@
+"""Generator of the LayerNorm backward kernels.
+
+The reference computes ``dx`` per row and accumulates ``dw``/``db`` partial sums into
+``GROUP_SIZE_M`` buffers of the weights' precision guarded by spin locks, then reduces those
+buffers (benchmarks/triton/layernorm_triton.py:206-311, host side :352-384).  The arithmetic here
+is the same -- ``xhat = (x-mean)*rstd``, ``wdy = w*dy``, ``c1 = mean(xhat*wdy)``, ``c2 = mean(wdy)``,
+``dx = (wdy - (xhat*c1 + c2))*rstd``, ``dw = sum(dy*xhat)``, ``db = sum(dy)`` -- but the partial sums
+stay in fp32 registers of a workgroup that walks several rows and are written once, so there
+is no lock and the summation order is fixed.  The LEGO offsets are the reference's:
+``N*pid + arange`` for x/dy/dx (``X_L['pid', 0, 0, :]``) and ``N*lock_id + arange`` for the
+partials (``X_L['lock_id', 0, 0, :]``), with the row dealt by ``Row(steps, G)``.
+"""
+from __future__ import annotations
+
+from ..lego import OrderBy, Row
+from .common import BANNER, Emitted, code, idx, size, template, tidy
+
+THREADS = 256
+MAX_GROUPS = 512      # workgroups of stage 1 = rows of the partial buffers
+VPTS = (1, 2, 4)      # 16-byte vectors per lane: rows of up to 8192 elements
+
+
+def emit():
+    M, N, G, STEPS = size("M"), size("N"), size("G"), size("STEPS")
+    wg, t, it, step, row, v = (idx(n) for n in ("wg", "t", "it", "step", "row", "v"))
+    rows = OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])
+    row_e = tidy(rows[step, wg], {step: (0, STEPS), wg: (0, G)})
+    X = OrderBy(Row(M, N)).TileBy([M, N / 8], [1, 8])
+    P = OrderBy(Row(G, N)).TileBy([G, N / 8], [1, 8])
+    params = dict(
+        banner=BANNER, THREADS=THREADS, WAVES=THREADS // 64, VPTS=list(VPTS), MAX_GROUPS=MAX_GROUPS,
+        row_layout="OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])[step, wg]",
+        x_layout="OrderBy(Row(M, N)).TileBy([M, N/8], [1, 8])[row, v, 0, :]",
+        part_layout="OrderBy(Row(G, N)).TileBy([G, N/8], [1, 8])[wg, v, 0, :]",
+        row=code(row_e),
+        row_base=code(tidy(X[row, 0, 0, 0], {row: (0, M)})).replace("row", "static_cast<size_t>(row)"),
+        vec=code(it * THREADS + t),
+        vec_off=code(tidy(X[0, v, 0, 0], {v: (0, N / 8)})),
+        stat_off=code(OrderBy(Row(M)).TileBy([M])[row,]),
+        part_off=code(tidy(P[wg, v, 0, 0], {wg: (0, G), v: (0, N / 8)})).replace("wg", "static_cast<size_t>(wg)"),
+    )
+    text = template("layernorm_bwd.hip.j2").render(**params)
+    return Emitted("layernorm_bwd_f16.hip", text, ["lego_layernorm_bwd_f16_launch"]), dict(
+        MAX_N=max(VPTS) * THREADS * 8, MAX_GROUPS=MAX_GROUPS)

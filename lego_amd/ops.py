@@ -97,11 +97,48 @@ def layer_norm_fwd(x, weight, bias, eps=1e-5, waves_per_row: int | None = None):
     return y.view(x.shape), mean, rstd
 
 
-def lego_layer_norm(x, normalized_shape, weight, bias, eps):
-    """Forward of the reference's ``lego_layer_norm`` (``LEGOLayerNorm.apply``)."""
-    if tuple(normalized_shape) != (x.shape[-1],):
-        raise ValueError("normalized_shape must be the last dimension of x")
-    return layer_norm_fwd(x, weight, bias, eps)[0]
+def layer_norm_bwd(dy, x, weight, mean, rstd):
+    """LayerNorm backward; returns ``(dx, dw, db)``.  fp16, rows of up to 8192 elements."""
+    x_arg = x.reshape(-1, x.shape[-1])
+    dy_arg = dy.reshape(-1, dy.shape[-1])
+    _check(x_arg, torch.float16, "x")
+    _check(dy_arg.contiguous(), torch.float16, "dy")
+    dy_arg = dy_arg.contiguous()
+    _check(weight, torch.float16, "weight", ndim=1)
+    M, N = x_arg.shape
+    need = ctypes.c_ulonglong(0)
+    runtime.call("lego_hip_layernorm_bwd_workspace_bytes", M, N, ctypes.byref(need))
+    # like the reference's wrapper, which allocates its partial buffers with torch (layernorm.py:381-383)
+    workspace = torch.empty(need.value // 4, dtype=torch.float32, device=x.device)
+    dx = torch.empty_like(x_arg)
+    dw = torch.empty((N,), dtype=weight.dtype, device=x.device)
+    db = torch.empty((N,), dtype=weight.dtype, device=x.device)
+    runtime.call("lego_hip_layernorm_bwd_f16", _ptr(dy_arg), _ptr(x_arg), _ptr(weight), _ptr(mean), _ptr(rstd),
+                 _ptr(dx), _ptr(dw), _ptr(db), _ptr(workspace), need, M, N, _stream())
+    return dx.view(x.shape), dw, db
+
+
+class LEGOLayerNorm(torch.autograd.Function):
+    """``lego_layer_norm = LEGOLayerNorm.apply`` with the reference's signature and gradients
+    (triton_generated/layernorm/layernorm.py:323-405)."""
+
+    @staticmethod
+    def forward(ctx, x, normalized_shape, weight, bias, eps):
+        if tuple(normalized_shape) != (x.shape[-1],):
+            raise ValueError("normalized_shape must be the last dimension of x")
+        y, mean, rstd = layer_norm_fwd(x, weight, bias, eps)
+        ctx.save_for_backward(x, weight, bias, mean, rstd)
+        ctx.eps = eps
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w, b, m, v = ctx.saved_tensors
+        dx, dw, db = layer_norm_bwd(dy, x, w, m, v)
+        return dx, None, dw, db, None
+
+
+lego_layer_norm = LEGOLayerNorm.apply
 
 
 def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "") -> torch.Tensor:

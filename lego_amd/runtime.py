@@ -31,6 +31,8 @@ SIGNATURES = {
     "lego_hip_softmax_f16_wpr": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "lego_hip_layernorm_fwd_f16_wpr": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                        _c_int, _c_int, _c_float, _c_int, _c_void_p],
+    "lego_hip_layernorm_bwd_workspace_bytes": [_c_int, _c_int, ctypes.POINTER(ctypes.c_ulonglong)],
+    "lego_hip_layernorm_bwd_f16": [_c_void_p] * 9 + [ctypes.c_ulonglong, _c_int, _c_int, _c_void_p],
     "lego_hip_copy16": [_c_void_p, _c_void_p, ctypes.c_ulonglong, _c_void_p],
 }
 

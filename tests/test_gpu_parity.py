@@ -155,6 +155,52 @@ def test_layernorm_reference_test_shape(ops):
     assert (got.float() - want.float()).abs().max().item() <= TOL
 
 
+def test_layernorm_backward_reference_test(ops):
+    """The reference's forward+backward test (layernorm.py:435-458): M=1151, N=8192, fp16,
+    y, dx, dw, db against torch autograd at atol=1e-2."""
+    print("layernorm backward reference test", flush=True)
+    from lego_amd.ops import lego_layer_norm
+    torch.manual_seed(0)
+    M, N = 1151, 8192
+    weight = torch.rand(N, dtype=torch.float16, device="cuda", requires_grad=True)
+    bias = torch.rand(N, dtype=torch.float16, device="cuda", requires_grad=True)
+    x = (-2.3 + 0.5 * torch.randn(M, N, dtype=torch.float16, device="cuda"))
+    dy = 0.1 * torch.randn_like(x)
+    x.requires_grad_(True)
+    y = lego_layer_norm(x, (N,), weight, bias, 1e-5)
+    y.backward(dy, retain_graph=True)
+    dx, dw, db = [t.grad.clone() for t in (x, weight, bias)]
+    x.grad, weight.grad, bias.grad = None, None, None
+    # the oracle: fp32 autograd on the CPU
+    xc, wc, bc = (t.detach().cpu().float().requires_grad_(True) for t in (x, weight, bias))
+    yr = torch.nn.functional.layer_norm(xc, (N,), wc, bc, 1e-5)
+    yr.backward(dy.cpu().float())
+    assert torch.allclose(y.detach().cpu().float(), yr.detach(), atol=1e-2, rtol=0)
+    assert torch.allclose(dx.cpu().float(), xc.grad, atol=1e-2, rtol=0)
+    assert (dx.cpu().float() - xc.grad).abs().max().item() <= TOL
+    # dw, db are sums over 1151 rows: compare relative to their magnitude (fp16 output)
+    assert torch.allclose(dw.cpu().float(), wc.grad, atol=1e-2, rtol=2e-3)
+    assert torch.allclose(db.cpu().float(), bc.grad, atol=1e-2, rtol=2e-3)
+
+
+@pytest.mark.parametrize("M,N", [(1, 8), (3, 520), (700, 1024), (513, 2048), (64, 8192)])
+def test_layernorm_backward_matches_oracle(ops, M, N):
+    print(f"layernorm backward {M}x{N}", flush=True)
+    g = _gen(6)
+    x = (2.0 * torch.randn(M, N, generator=g)).half()
+    w = (1 + 0.1 * torch.randn(N, generator=g)).half()
+    b = (0.1 * torch.randn(N, generator=g)).half()
+    dy = (0.1 * torch.randn(M, N, generator=g)).half()
+    _, mean, rstd = ops.layer_norm_fwd(x.cuda(), w.cuda(), b.cuda(), 1e-5)
+    dx, dw, db = ops.layer_norm_bwd(dy.cuda(), x.cuda(), w.cuda(), mean, rstd)
+    xc, wc, bc = (t.float().requires_grad_(True) for t in (x, w, b))
+    torch.nn.functional.layer_norm(xc, (N,), wc, bc, 1e-5).backward(dy.float())
+    assert (dx.cpu().float() - xc.grad).abs().max().item() <= TOL
+    scale = max(1.0, wc.grad.abs().max().item())
+    assert (dw.cpu().float() - wc.grad).abs().max().item() <= 2e-3 * scale
+    assert (db.cpu().float() - bc.grad).abs().max().item() <= 2e-3 * max(1.0, bc.grad.abs().max().item())
+
+
 def test_config3_full_size(ops):
     print("config 3 full size", flush=True)
     g = _gen(2)
