@@ -62,6 +62,9 @@ int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, con
  * Like the reference kernel (no edge masks, matmul_sympy.py:196-203) the sizes must divide
  * the tiles: M and N multiples of 256, K a multiple of 64. */
 int lego_hip_gemm_f16(const void* a, const void* b, void* c, int M, int N, int K, void* stream);
+/* The same with the reference's fused epilogue (matmul(a, b, activation="leaky_relu"),
+ * matmul_NTA_NTB.py:129-145): activation 0 = none, 1 = leaky_relu on the fp32 accumulator. */
+int lego_hip_gemm_f16_act(const void* a, const void* b, void* c, int M, int N, int K, int activation, void* stream);
 
 /* groups independent GEMMs in one launch.  a, b, c are HOST arrays of `groups` device
  * pointers; sizes3 is a HOST array of groups*3 ints (M, N, K per problem).  At most 64

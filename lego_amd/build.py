@@ -82,7 +82,7 @@ def generate():
           "hipError_t lego_layernorm_bwd_f16_launch(const void*, const void*, const void*, const float*, const float*, "
           "void*, void*, void*, float*, int, int, hipStream_t);",
           f"#define LEGO_LAYERNORM_BWD_MAX_N {mlb['MAX_N']}", ""]
-    h += ["hipError_t lego_gemm_f16_launch(const void*, const void*, void*, int, int, int, hipStream_t);",
+    h += ["hipError_t lego_gemm_f16_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);",
           "hipError_t lego_grouped_gemm_f16_launch(const void* const*, const void* const*, void* const*, "
           "const int*, int, hipStream_t);",
           f"#define LEGO_GEMM_BM {mg['BM']}", f"#define LEGO_GEMM_BN {mg['BN']}", f"#define LEGO_GEMM_BK {mg['BK']}",

@@ -143,8 +143,8 @@ lego_layer_norm = LEGOLayerNorm.apply
 
 def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "") -> torch.Tensor:
     """``a @ b`` for row-major fp16 operands, fp32 accumulation, fp16 result."""
-    if activation != "":
-        raise NotImplementedError("fused activations are not generated by this build")
+    if activation not in ("", "leaky_relu"):
+        raise NotImplementedError(f"activation {activation!r} is not generated by this build")
     _check(a, torch.float16, "a")
     _check(b, torch.float16, "b")
     M, K = a.shape
@@ -152,7 +152,7 @@ def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "") -> torch.Tens
     if K != K2:
         raise ValueError("Incompatible dimensions")
     c = torch.empty((M, N), device=a.device, dtype=torch.float16)
-    runtime.call("lego_hip_gemm_f16", _ptr(a), _ptr(b), _ptr(c), M, N, K, _stream())
+    runtime.call("lego_hip_gemm_f16_act", _ptr(a), _ptr(b), _ptr(c), M, N, K, 1 if activation else 0, _stream())
     return c
 
 

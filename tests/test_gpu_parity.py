@@ -271,4 +271,16 @@ def test_gemm_rejects_bad_shapes(ops):
                    torch.zeros(64, 256, device="cuda", dtype=torch.half))
     with pytest.raises(NotImplementedError):
         ops.matmul(torch.zeros(256, 64, device="cuda", dtype=torch.half),
-                   torch.zeros(64, 256, device="cuda", dtype=torch.half), activation="leaky_relu")
+                   torch.zeros(64, 256, device="cuda", dtype=torch.half), activation="gelu")
+
+
+def test_gemm_leaky_relu_epilogue(ops):
+    print("gemm leaky_relu", flush=True)
+    g = _gen(8)
+    a = (torch.randn(512, 256, generator=g) / 16).half()
+    b = (torch.randn(256, 512, generator=g) / 16).half()
+    want = torch.nn.functional.leaky_relu(a.float() @ b.float(), 0.01).half()
+    got = ops.matmul(a.cuda(), b.cuda(), activation="leaky_relu").cpu()
+    assert _rel_err(got, want) <= 1e-2
+    assert (got.float() - want.float()).abs().max().item() <= 1e-2
+    assert (got < 0).any() and (got > 0).any()
