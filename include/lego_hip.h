@@ -65,6 +65,11 @@ int lego_hip_gemm_f16(const void* a, const void* b, void* c, int M, int N, int K
 /* The same with the reference's fused epilogue (matmul(a, b, activation="leaky_relu"),
  * matmul_NTA_NTB.py:129-145): activation 0 = none, 1 = leaky_relu on the fp32 accumulator. */
 int lego_hip_gemm_f16_act(const void* a, const void* b, void* c, int M, int N, int K, int activation, void* stream);
+/* The reference's four operand layouts (matmul_{N,}TA_{N,}TB.py: the operands there are `.T`
+ * views, i.e. column-major storage of the same logical matrices): trans_a != 0 means `a` points
+ * to a K x M row-major buffer, trans_b != 0 means `b` points to an N x K row-major buffer. */
+int lego_hip_gemm_f16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
+                         int activation, void* stream);
 
 /* groups independent GEMMs in one launch.  a, b, c are HOST arrays of `groups` device
  * pointers; sizes3 is a HOST array of groups*3 ints (M, N, K per problem).  At most 64

@@ -53,8 +53,10 @@ def generate():
             units.append(unit)
             tmeta.setdefault(dtype, []).append(meta)
     units += [rowwise.emit(w, dtype, vec) for dtype, vec, w in ROWWISE]
-    g, mg = gemm.emit(**GEMM)
-    units.append(g)
+    for ta in (False, True):
+        for tb in (False, True):
+            g, mg = gemm.emit(**GEMM, trans_a=ta, trans_b=tb, with_grouped=not (ta or tb))
+            units.append(g)
     lb, mlb = layernorm_bwd.emit()
     units.append(lb)
 
@@ -82,7 +84,9 @@ def generate():
           "hipError_t lego_layernorm_bwd_f16_launch(const void*, const void*, const void*, const float*, const float*, "
           "void*, void*, void*, float*, int, int, hipStream_t);",
           f"#define LEGO_LAYERNORM_BWD_MAX_N {mlb['MAX_N']}", ""]
-    h += ["hipError_t lego_gemm_f16_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);",
+    h += [f"hipError_t lego_gemm_f16_{v}_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);"
+          for v in ("nn", "nt", "tn", "tt")]
+    h += [
           "hipError_t lego_grouped_gemm_f16_launch(const void* const*, const void* const*, void* const*, "
           "const int*, int, hipStream_t);",
           f"#define LEGO_GEMM_BM {mg['BM']}", f"#define LEGO_GEMM_BN {mg['BN']}", f"#define LEGO_GEMM_BK {mg['BK']}",

@@ -126,17 +126,27 @@ int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, con
                                              as_stream(stream)));
 }
 
-int lego_hip_gemm_f16_act(const void* a, const void* b, void* c, int M, int N, int K, int activation, void* stream)
+int lego_hip_gemm_f16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
+                         int activation, void* stream)
 {
   if (!usable(a) || !usable(b) || !usable(c)) return kInvalid;
   if (M <= 0 || N <= 0 || K <= 0 || M % LEGO_GEMM_BM || N % LEGO_GEMM_BN || K % LEGO_GEMM_BK) return kInvalid;
   if (activation != 0 && activation != 1) return kInvalid;
-  return ok_or(lego_gemm_f16_launch(a, b, c, M, N, K, activation, as_stream(stream)));
+  hipStream_t s = as_stream(stream);
+  if (!trans_a && !trans_b) return ok_or(lego_gemm_f16_nn_launch(a, b, c, M, N, K, activation, s));
+  if (!trans_a && trans_b) return ok_or(lego_gemm_f16_nt_launch(a, b, c, M, N, K, activation, s));
+  if (trans_a && !trans_b) return ok_or(lego_gemm_f16_tn_launch(a, b, c, M, N, K, activation, s));
+  return ok_or(lego_gemm_f16_tt_launch(a, b, c, M, N, K, activation, s));
+}
+
+int lego_hip_gemm_f16_act(const void* a, const void* b, void* c, int M, int N, int K, int activation, void* stream)
+{
+  return lego_hip_gemm_f16_ex(a, b, c, M, N, K, 0, 0, activation, stream);
 }
 
 int lego_hip_gemm_f16(const void* a, const void* b, void* c, int M, int N, int K, void* stream)
 {
-  return lego_hip_gemm_f16_act(a, b, c, M, N, K, 0, stream);
+  return lego_hip_gemm_f16_ex(a, b, c, M, N, K, 0, 0, 0, stream);
 }
 
 int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* const* c,

@@ -97,7 +97,7 @@ def xcd_remap(per, wg, xcds=XCDS):
     return OrderBy(Col(per, xcds)).TileBy([per, xcds])[j, x]
 
 
-def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
+def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, trans_b=False, with_grouped=True):
     WAVES_M, WAVES_N = waves
     THREADS = 64 * WAVES_M * WAVES_N
     WM, WN = bm // WAVES_M, bn // WAVES_N
@@ -116,11 +116,16 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
     wm, wn, l32, lhi, l16, lgrp = (idx(n) for n in ("wm", "wn", "l32", "lhi", "l16", "lgrp"))
     cr, cc = idx("cr"), idx("cc")
 
-    A_L = OrderBy(Row(M, K)).TileBy([M / bm, K / bk], [bm, bk])
-    B_L = OrderBy(Row(K, N)).TileBy([K / bk, N / bn], [bk, bn])
+    # the reference's operand layouts with its transpose flags (matmul_sympy.py:37-46): a transposed
+    # operand is the column-major layout of the same logical matrix
+    A_L = OrderBy(Col(M, K) if trans_a else Row(M, K)).TileBy([M / bm, K / bk], [bm, bk])
+    B_L = OrderBy(Col(K, N) if trans_b else Row(K, N)).TileBy([K / bk, N / bn], [bk, bn])
     C_L = OrderBy(Row(M, N)).TileBy([M / bm, N / bn], [bm, bn])
-    As_L = lds_a_layout(bm, bk // 8)
-    Bs_L = lds_b_layout(bk, bn)
+    # An operand tile is "k-major" when its k-values are contiguous in memory (A as given, B
+    # transposed): it is staged as [row][16-byte chunk of k] and a fragment is one 16-byte read.
+    # Otherwise (B as given, A transposed) it is staged as in memory, [k][row], and a fragment is
+    # two transposing 8-byte reads.
+    a_kmajor, b_kmajor = not trans_a, trans_b
 
     wm_e, wn_e = OrderBy(Row(WAVES_M, WAVES_N)).TileBy([WAVES_M, WAVES_N]).inv(wave)
 
@@ -155,9 +160,6 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
     c_out = [tidy(e, {lane_o: (0, 64), it: (0, WM * WN // 8 // 64)}) for e in
              OrderBy(Row(WM, WN // 8)).TileBy([WM, WN // 8]).inv(it * 64 + lane_o)]
 
-    frag_row = wm * WM + i * 32 + l32
-    frag_k = [ks * 16 + (lgrp // 2) * 8 + h * 4 + l16 // 4 for h in (0, 1)]
-    frag_n = wn * WN + j * 32 + (lgrp % 2) * 16 + 4 * (l16 % 4)
     pm_e, pn_e = launch_order(npm, npn, group_m, pid)
 
     # memory->LDS: instruction `it` of wave `wave` fills slots (it*WAVES + wave)*64 + lane; the chunk
@@ -166,17 +168,42 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
     lane_s = idx("lane")
     slot = (it * WAVES + wave) * 64 + lane_s
     slot_rng = {lane_s: (0, 64), wave: (0, WAVES), it: (0, max(A_ITERS, B_ITERS))}
-    a_row, a_ch = (tidy(e, slot_rng) for e in As_L.inv(slot))
-    b_kr, b_n = (tidy(e, slot_rng) for e in Bs_L.inv(8 * slot))
-    b_ch = tidy(b_n / 8, slot_rng)
-    sub_a = {row: a_row, ch: a_ch}
-    sub_b = {kr: b_kr, ch: b_ch}
-    a_full = tidy(A_L[pid_m, k, row, ch * 8], rng)     # the reference's a_ptrs expression
-    b_full = tidy(B_L[k, pid_n, kr, ch * 8], rng)     # and its b_ptrs expression
-    a_src0, a_src_step = chunk_walk(a_full.subs({pid_m: 0, k: 0}).subs(sub_a), A_ITERS)
-    b_src0, b_src_step = chunk_walk(b_full.subs({pid_n: 0, k: 0}).subs(sub_b), B_ITERS)
-    chunk_params = dict(a_src0=code(a_src0), a_src_step=code(a_src_step), b_src0=code(b_src0),
-                        b_src_step=code(b_src_step), WAVES=WAVES)
+
+    def operand(role):
+        """Everything the template needs for operand ``role``: where a lane's memory->LDS chunk
+        comes from, the k-tile stride, and the text that reads one MFMA fragment."""
+        kmajor = a_kmajor if role == "a" else b_kmajor
+        rows, tile_id = (bm, pid_m) if role == "a" else (bn, pid_n)
+        wave_off, sub = (wm * WM + i * 32, i) if role == "a" else (wn * WN + j * 32, j)
+        n_iters = A_ITERS if role == "a" else B_ITERS
+
+        def glob(row_e, kk_e):   # offset of element (row, kk) of k-tile k of this operand's tile
+            return A_L[pid_m, k, row_e, kk_e] if role == "a" else B_L[k, pid_n, kk_e, row_e]
+
+        if kmajor:
+            lds = lds_a_layout(rows, bk // 8)
+            r_e, ch_e = (tidy(e, slot_rng) for e in lds.inv(slot))
+            full = tidy(glob(row, ch * 8), rng)
+            placed = full.subs({row: r_e, ch: ch_e})
+            frag = ("*reinterpret_cast<const half8*>(%ss + (%s))"
+                    % (role, code(tidy(8 * lds[wave_off + l32, ks * 2 + lhi], rng))))
+        else:
+            lds = lds_b_layout(bk, rows)
+            kr_e, col_e = (tidy(e, slot_rng) for e in lds.inv(8 * slot))
+            full = tidy(glob(8 * ch, kr), rng)      # here `ch` counts 8-element chunks along the row
+            placed = full.subs({kr: kr_e, ch: tidy(col_e / 8, slot_rng)})
+            frag_k = [ks * 16 + (lgrp // 2) * 8 + h * 4 + l16 // 4 for h in (0, 1)]
+            frag_c = wave_off + (lgrp % 2) * 16 + 4 * (l16 % 4)
+            frag = ("read_b_fragment(%ss + (%s), %ss + (%s))"
+                    % (role, code(tidy(lds[frag_k[0], frag_c], rng)), role, code(tidy(lds[frag_k[1], frag_c], rng))))
+        src0, step = chunk_walk(placed.subs({tile_id: 0, k: 0}), n_iters)
+        return {f"{role}_src0": code(src0), f"{role}_src_step": code(step),
+                f"{role}_goff_base": code(full.subs({k: 0, row: 0, ch: 0, kr: 0})),
+                f"{role}_kstep": code(sp.simplify(full.subs(k, k + 1) - full)),
+                f"{role}_frag_code": frag}
+
+    variant = ("t" if trans_a else "n") + ("t" if trans_b else "n")
+    chunk_params = dict(WAVES=WAVES, variant=variant, with_grouped=with_grouped, **operand("a"), **operand("b"))
 
     params = dict(
         banner=BANNER, BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
@@ -184,19 +211,13 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
         pid_layout="OrderBy(Col(max(npm//GM,1),1), Col(min(npm,GM),npn)).TileBy([npm,npn]).inv(pid)",
         MAX_GM=max_group_m,
         xcd_layout=f"OrderBy(Col(nwg/{XCDS}, {XCDS})).TileBy([nwg/{XCDS}, {XCDS}])[Row(nwg/{XCDS}, {XCDS}).inv(wg)]",
-        a_layout=f"OrderBy(Row(M,K)).TileBy([M/{bm},K/{bk}],[{bm},{bk}])",
-        b_layout=f"OrderBy(Row(K,N)).TileBy([K/{bk},N/{bn}],[{bk},{bn}])",
+        a_layout=f"OrderBy({'Col' if trans_a else 'Row'}(M,K)).TileBy([M/{bm},K/{bk}],[{bm},{bk}])",
+        b_layout=f"OrderBy({'Col' if trans_b else 'Row'}(K,N)).TileBy([K/{bk},N/{bn}],[{bk},{bn}])",
+        a_kmajor=a_kmajor, b_kmajor=b_kmajor,
         c_layout=f"OrderBy(Row(M,N)).TileBy([M/{bm},N/{bn}],[{bm},{bn}])",
         wm=code(wm_e), wn=code(wn_e),
         # offset of a chunk = tile base (uniform) + position inside k-tile 0 (per lane) + k * step
         **chunk_params,
-        a_goff_base=code(a_full.subs({k: 0, row: 0, ch: 0})),
-        b_goff_base=code(b_full.subs({k: 0, kr: 0, ch: 0})),
-        a_kstep=code(sp.simplify(a_full.subs(k, k + 1) - a_full)),
-        b_kstep=code(sp.simplify(b_full.subs(k, k + 1) - b_full)),
-        a_frag=code(tidy(8 * As_L[frag_row, ks * 2 + lhi], rng)),
-        b_frag0=code(tidy(Bs_L[frag_k[0], frag_n], rng)),
-        b_frag1=code(tidy(Bs_L[frag_k[1], frag_n], rng)),
         # accumulator -> staging: row i*32 + l32, 8-byte chunk (j*32 + q*8 + lhi*4)/4 of the wave's block
         c_stage_store=code(tidy(4 * Cs_L[i * 32 + l32, j * 8 + q * 2 + lhi], rng)),
         # staging -> memory: lane reads the pair of chunks (2p, 2p+1) of row cr; the XOR keeps a
@@ -209,4 +230,5 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8):
     )
     text = template("gemm.hip.j2").render(**params)
     meta = dict(BM=bm, BN=bn, BK=bk, MAX_GROUPS=MAX_GROUPS)
-    return Emitted("gemm_f16.hip", text, ["lego_gemm_f16_launch", "lego_grouped_gemm_f16_launch"]), meta
+    launchers = [f"lego_gemm_f16_{variant}_launch"] + (["lego_grouped_gemm_f16_launch"] if with_grouped else [])
+    return Emitted(f"gemm_f16_{variant}.hip", text, launchers), meta

@@ -141,18 +141,32 @@ class LEGOLayerNorm(torch.autograd.Function):
 lego_layer_norm = LEGOLayerNorm.apply
 
 
+def _operand(t, name):
+    """``(storage tensor, transposed?)`` of a 2-D fp16 operand that is contiguous either as given
+    or as its transpose (the reference's TA/TB variants pass ``x.T`` views)."""
+    if not t.is_cuda or t.dtype != torch.float16 or t.dim() != 2:
+        raise ValueError(f"{name} must be a 2-D float16 GPU tensor")
+    if t.is_contiguous():
+        return t, 0
+    if t.t().is_contiguous():
+        return t.t(), 1
+    raise ValueError(f"{name} must be contiguous or the transpose of a contiguous tensor")
+
+
 def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "") -> torch.Tensor:
-    """``a @ b`` for row-major fp16 operands, fp32 accumulation, fp16 result."""
+    """``act(a @ b)`` for fp16 operands, each row-major or column-major (a ``.T`` view), fp32
+    accumulation, fp16 row-major result."""
     if activation not in ("", "leaky_relu"):
         raise NotImplementedError(f"activation {activation!r} is not generated by this build")
-    _check(a, torch.float16, "a")
-    _check(b, torch.float16, "b")
+    a_store, ta = _operand(a, "a")
+    b_store, tb = _operand(b, "b")
     M, K = a.shape
     K2, N = b.shape
     if K != K2:
         raise ValueError("Incompatible dimensions")
     c = torch.empty((M, N), device=a.device, dtype=torch.float16)
-    runtime.call("lego_hip_gemm_f16_act", _ptr(a), _ptr(b), _ptr(c), M, N, K, 1 if activation else 0, _stream())
+    runtime.call("lego_hip_gemm_f16_ex", _ptr(a_store), _ptr(b_store), _ptr(c), M, N, K, ta, tb,
+                 1 if activation else 0, _stream())
     return c
 
 

@@ -274,6 +274,36 @@ def test_gemm_rejects_bad_shapes(ops):
                    torch.zeros(64, 256, device="cuda", dtype=torch.half), activation="gelu")
 
 
+@pytest.mark.parametrize("ta,tb", [(False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 768, 320), (1024, 256, 1024)])
+def test_gemm_transposed_operands(ops, ta, tb, M, N, K):
+    """The reference's TA/TB variants: operands are .T views of contiguous tensors."""
+    print(f"gemm ta={ta} tb={tb} {M}x{N}x{K}", flush=True)
+    g = _gen(9)
+    a = (torch.randn(M, K, generator=g) / math.sqrt(K)).half()
+    b = (torch.randn(K, N, generator=g) / math.sqrt(K)).half()
+    want = ok.gemm(a, b)
+    ad = a.t().contiguous().cuda().t() if ta else a.cuda()
+    bd = b.t().contiguous().cuda().t() if tb else b.cuda()
+    assert ad.shape == (M, K) and bd.shape == (K, N)
+    got = ops.matmul(ad, bd).cpu()
+    assert _rel_err(got, want) <= 1e-2
+    assert (got.float() - want.float()).abs().max().item() <= 1e-2
+
+
+def test_gemm_transposed_integer_exact(ops):
+    g = _gen(10)
+    a = torch.randint(-2, 3, (512, 256), generator=g).half()
+    b = torch.randint(-2, 3, (256, 768), generator=g).half()
+    want = a.double() @ b.double()
+    for ta in (False, True):
+        for tb in (False, True):
+            print(f"gemm integer exact ta={ta} tb={tb}", flush=True)
+            ad = a.t().contiguous().cuda().t() if ta else a.cuda()
+            bd = b.t().contiguous().cuda().t() if tb else b.cuda()
+            assert torch.equal(ops.matmul(ad, bd).cpu().double(), want)
+
+
 def test_gemm_leaky_relu_epilogue(ops):
     print("gemm leaky_relu", flush=True)
     g = _gen(8)
