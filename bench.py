@@ -27,9 +27,9 @@ import time
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/transpose_f16_16384_pmc.txt); None until measured.
-HEADLINE_TRAFFIC_BYTES = None
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
+# what the same counters read for lego_hip_copy16 on 512 MiB (profiles/hbm_traffic_pmc.txt).
+HEADLINE_TRAFFIC_BYTES = 1073755391
 
 
 def main():
@@ -38,7 +38,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of configs to time (c1,c2,c3,c4,c5)")
+    ap.add_argument("--only", default="", help="comma list of configs to time (c1,c2,c3,c4,c5,extra); "
+                    "c2 is always timed; 'extra' adds LayerNorm backward and the transposed GEMM layouts")
     ns = ap.parse_args()
     if ns.gpus != 1:
         print("bench.py: this build measures one MI355X; every configuration of the hot path is a "
@@ -162,6 +163,24 @@ def main():
                                  frac_hbm=by3 / rot / 1e6 / HBM_PEAK_GBS, bytes=by3, max_abs_err_vs_fp32=err,
                                  note="gbs = rotating buffers (1 GiB pool); gbs_hot = cache resident; "
                                       "x ~ N(0, sigma=2)")
+        # next row: LayerNorm backward (reference formula: 3 * numel * element size, layernorm.py:555)
+        if want("extra"):
+            dy3 = (0.1 * torch.randn(m3, n3, generator=gen(6))).half().to(dev)
+            ln()
+            torch.cuda.synchronize()
+            need = ctypes.c_ulonglong(0)
+            runtime.call("lego_hip_layernorm_bwd_workspace_bytes", m3, n3, ctypes.byref(need))
+            ws = torch.empty(need.value // 4, device=dev)
+            dx3, dw3, db3 = torch.empty_like(x3), torch.empty_like(w3), torch.empty_like(b3)
+
+            def lnb():
+                runtime.call("lego_hip_layernorm_bwd_f16", p(dy3), p(x3), p(w3), p(mean3), p(rstd3), p(dx3), p(dw3),
+                             p(db3), p(ws), need, m3, n3, stream)
+            ms_b = timed(lnb)
+            kernels["next_layernorm_bwd_f16_8192"] = dict(ms=ms_b, gbs=3 * m3 * n3 * 2 / ms_b / 1e6,
+                                                         frac_hbm=3 * m3 * n3 * 2 / ms_b / 1e6 / HBM_PEAK_GBS,
+                                                         bytes=3 * m3 * n3 * 2, note="cache-resident buffers")
+            del dy3, dx3, ws
         del x3, y3
 
     # ---- C4: fp16 GEMM 8192^3 ----------------------------------------------------------------------
@@ -185,6 +204,13 @@ def main():
                                            flop=fl4, rel_err_vs_fp32=rel,
                                            vendor_library_tflops=fl4 / lib_ms / 1e9,
                                            note="vendor_library = torch.matmul (hipBLASLt) on the same buffers")
+        if want("extra"):
+            for ta, tb in ((0, 1), (1, 0), (1, 1)):
+                def gv(ta=ta, tb=tb):
+                    runtime.call("lego_hip_gemm_f16_ex", p(a4), p(b4), p(c4), n4, n4, n4, ta, tb, 0, stream)
+                msv = timed(gv, steps=max(5, K // 5), warmup=max(2, W // 5))
+                kernels[f"next_gemm_f16_8192_{'t' if ta else 'n'}{'t' if tb else 'n'}"] = dict(
+                    ms=msv, tflops=fl4 / msv / 1e9, frac_mfma=fl4 / msv / 1e9 / MFMA_F16_PEAK_TFLOPS)
         del a4, b4, c4, ref
 
     # ---- C5: grouped fp16 GEMM, 8 problems -------------------------------------------------------------
