@@ -259,11 +259,11 @@ def main():
         "value": gbs2, "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": ms2,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "2-D fp16 transpose 16384x16384, LEGO TileBy([256,256],[64,64]) row-major -> "
-                               "column-major, 1x4 tiles per workgroup in skewed order, XOR-swizzled LDS "
+                               "column-major, 1x4 tiles per workgroup, workgroups in windows of 128x8 macro tiles, XOR-swizzled LDS "
                                "staging, inputs N(0,1) seed 1"},
         "roofline": {"bound": "hbm", "achieved": gbs2, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs2 / HBM_PEAK_GBS, "traffic": HEADLINE_TRAFFIC_BYTES,
-                     "kernel": "lego_transpose_f16_64x256", "algorithmic_bytes_per_launch": bytes2},
+                     "kernel": "lego_transpose_f16_64x256_w128x8", "algorithmic_bytes_per_launch": bytes2},
         "cpu_baseline": cpu,
         "kernels": kernels,
         "peaks": {"hbm_gbs": HBM_PEAK_GBS, "mfma_f16_tflops": MFMA_F16_PEAK_TFLOPS},

@@ -30,7 +30,8 @@ OBJ_DIR = LIB_DIR / "obj"
 TRANSPOSE = {
     "f32": [dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag"),
             dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag")],
-    "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag"),
+    "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 128, 8)),
+            dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag"),
             dict(dtype="f16", tile=(64, 64), group=(1, 1), order="diag")],
 }
 # (element type, vectorised, waves per row): 16-byte accesses need N % (16/size) == 0; the
@@ -49,7 +50,7 @@ def generate():
     for dtype, configs in TRANSPOSE.items():
         for cfg in configs:
             unit, meta = transpose.emit(**cfg, suffix="")
-            unit.filename = f"transpose_{dtype}_{meta['SR']}x{meta['SC']}.hip"
+            unit.filename = meta["kernel"].replace("lego_", "", 1) + ".hip"
             units.append(unit)
             tmeta.setdefault(dtype, []).append(meta)
     units += [rowwise.emit(w, dtype, vec) for dtype, vec, w in ROWWISE]
@@ -68,7 +69,7 @@ def generate():
               f"inline hipError_t lego_transpose_{dtype}_dispatch(const void* in, void* out, int rows, int cols, "
               "hipStream_t stream) {"]
         for m in metas:
-            h.append(f"  if (rows % {m['SR']} == 0 && cols % {m['SC']} == 0) "
+            h.append(f"  if (rows % {m['row_multiple']} == 0 && cols % {m['col_multiple']} == 0) "
                      f"return {m['kernel']}_launch(in, out, rows, cols, stream);")
         h += ["  return hipErrorInvalidValue;", "}", ""]
     for dtype, vec, w in ROWWISE:

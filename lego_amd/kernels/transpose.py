@@ -108,7 +108,9 @@ def tile_order(order, n_bi, n_bj, wg):
     ``col``: the transpose of that (strided reads, contiguous writes);
     ``diag``: row order skewed by the tile row, ``Bj = (j + Bi) % n_bj``, so that workgroups
     that run together spread both their reads and their writes over tile columns -- the
-    classic remedy for DRAM channel camping when the row pitch is a power of two.
+    classic remedy for DRAM channel camping when the row pitch is a power of two;
+    ``("window", ti, tj)``: row order inside windows of ``ti x tj`` tiles, windows in row
+    order; ``n_bi`` and ``n_bj`` must be multiples of ``ti`` and ``tj``.
     """
     if order == "row":
         return OrderBy(Row(n_bi, n_bj)).TileBy([n_bi, n_bj]).inv(wg)
@@ -119,6 +121,14 @@ def tile_order(order, n_bi, n_bj, wg):
                     lambda ij: ij[0] * n_bj + (ij[1] - ij[0]) % n_bj,
                     lambda f: (f // n_bj, (f % n_bj + f // n_bj) % n_bj))
         return OrderBy(skew).TileBy([n_bi, n_bj]).inv(wg)
+    if isinstance(order, tuple) and order[0] == "window":
+        # windows of ti x tj tiles, row-major inside and across: with a window about as large
+        # as the set of workgroups in flight, the reads of that set are tj tiles wide per row
+        # and its writes ti tiles wide per output row, so both sides keep DRAM pages open
+        _, ti, tj = order
+        windows = OrderBy(Row(n_bi / ti, n_bj / tj), Row(ti, tj)).TileBy([n_bi / ti, n_bj / tj], [ti, tj])
+        wi, wj, i, j = windows.inv(wg)
+        return wi * ti + i, wj * tj + j
     raise ValueError(order)
 
 
@@ -150,7 +160,16 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix=""):
 
     # workgroup -> macro tile, row-major over the grid of macro tiles
     nBi, nBj = size("nBi"), size("nBj")
-    Bi_e, Bj_e = tile_order(order, nBi, nBj, wg)
+    windowed = isinstance(order, tuple)
+    if windowed:
+        # tile counts as multiples of the window, so that every division is exact
+        WI, WJ = order[1:]
+        Bi_e, Bj_e = tile_order(order, WI * size("nWi"), WJ * size("nWj"), wg)
+        Bi_e, Bj_e = tidy(Bi_e, {}), tidy(Bj_e, {})
+        suffix = f"_w{WI}x{WJ}{suffix}"
+    else:
+        WI = WJ = 1
+        Bi_e, Bj_e = tile_order(order, nBi, nBj, wg)
     # lane -> vector of the macro tile, phase 1
     W = SC // vec
     v1 = [tidy(x, {t: (0, THREADS), it: (0, P1)}) for x in phase1_vector(SR, W, esize, it, t)]
@@ -167,7 +186,7 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix=""):
         src_layout=f"OrderBy(Row(R, C)).TileBy([R/{SR}, C/{SC}], [{MR}, {MC}], [{TR}, {TC}])",
         dst_layout=f"OrderBy(Col(R, C)).TileBy([R/{SR}, C/{SC}], [{MR}, {MC}], [{TR}, {TC}])",
         lds_layout=f"OrderBy(GenP(({KD}, {SR}), xor-rotated rows)).TileBy([{KD}, {SR}])",
-        Bi=code(Bi_e), Bj=code(Bj_e),
+        Bi=code(Bi_e), Bj=code(Bj_e), WI=WI, WJ=WJ, windowed=windowed,
         p1_r=code(v1[0]), p1_cv=code(v1[1]),
         src_off=code(in_tile(src, r, cv * vec, rng1)),
         lds_store=code(tidy(lds[cv * 4 + e, r], rng1)),
@@ -180,4 +199,4 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix=""):
     )
     text = template("transpose.hip.j2").render(**params)
     return Emitted(f"transpose_{dtype}{suffix}.hip", text, [params["kernel"] + "_launch"]), dict(
-        SR=SR, SC=SC, kernel=params["kernel"])
+        SR=SR, SC=SC, kernel=params["kernel"], row_multiple=SR * WI, col_multiple=SC * WJ)

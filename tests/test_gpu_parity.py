@@ -27,6 +27,7 @@ def _gen(seed):
     (torch.float32, 64, 64), (torch.float32, 128, 320), (torch.float32, 1024, 512), (torch.float32, 32, 256),
     (torch.float32, 96, 768), (torch.float16, 64, 64), (torch.float16, 192, 128), (torch.float16, 512, 1024),
     (torch.float16, 64, 256), (torch.float16, 320, 768),
+    (torch.float16, 8192, 2048),                    # one window of the windowed tile order
 ])
 def test_transpose_matches_oracle(ops, dtype, rows, cols):
     print(f"transpose {dtype} {rows}x{cols}", flush=True)
@@ -51,6 +52,16 @@ def test_transpose_config2_fp16_16384_properties(ops):
     y = ops.transpose(x)
     assert torch.equal(y, x.t())
     assert torch.equal(ops.transpose(y), x)
+
+
+def test_transpose_windowed_order_rectangular(ops):
+    """Several windows per side, more across than down: a mix-up of the window digits
+    would move tiles."""
+    print("transpose fp16 16384x6144 (windowed order)", flush=True)
+    x = torch.randn(16384, 6144, generator=_gen(2)).half().cuda()
+    y = ops.transpose(x)
+    assert y.shape == (6144, 16384)
+    assert torch.equal(y, x.t())
 
 
 def test_transpose_rejects_bad_shapes(ops):
