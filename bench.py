@@ -29,7 +29,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
 # what the same counters read for lego_hip_copy16 on 512 MiB (profiles/hbm_traffic_pmc.txt).
-HEADLINE_TRAFFIC_BYTES = 1073755391
+HEADLINE_TRAFFIC_BYTES = 1074096255
 
 
 def main():
