@@ -24,11 +24,12 @@ LIB_PATH = LIB_DIR / "liblego_hip.so"
 OBJ_DIR = LIB_DIR / "obj"
 
 # the tilings the library is built with
-# Two tilings per element type: a wide macro tile (long read segments; fastest on MI355X) and a
-# 64x64 one for shapes the wide tile does not divide.  Tiles are dealt to workgroups in the
-# skewed ("diag") order.
+# Per element type, in order of preference: the fastest tiling for shapes that its windows
+# divide, a wide macro tile in skewed ("diag") order, and a 64x64 one for shapes the wide tile
+# does not divide.
 TRANSPOSE = {
-    "f32": [dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag"),
+    "f32": [dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 32, 8), max_bytes=256 << 20),
+            dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag"),
             dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag")],
     "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 128, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag"),
@@ -49,7 +50,10 @@ def generate():
     tmeta = {}
     for dtype, configs in TRANSPOSE.items():
         for cfg in configs:
+            cfg = dict(cfg)
+            max_bytes = cfg.pop("max_bytes", None)   # only for matrices that fit the last-level cache
             unit, meta = transpose.emit(**cfg, suffix="")
+            meta["max_bytes"] = max_bytes
             unit.filename = meta["kernel"].replace("lego_", "", 1) + ".hip"
             units.append(unit)
             tmeta.setdefault(dtype, []).append(meta)
@@ -69,7 +73,9 @@ def generate():
               f"inline hipError_t lego_transpose_{dtype}_dispatch(const void* in, void* out, int rows, int cols, "
               "hipStream_t stream) {"]
         for m in metas:
-            h.append(f"  if (rows % {m['row_multiple']} == 0 && cols % {m['col_multiple']} == 0) "
+            fits = "" if m["max_bytes"] is None else \
+                f" && 2ull * rows * cols * {4 if dtype == 'f32' else 2} <= {m['max_bytes']}ull"
+            h.append(f"  if (rows % {m['row_multiple']} == 0 && cols % {m['col_multiple']} == 0{fits}) "
                      f"return {m['kernel']}_launch(in, out, rows, cols, stream);")
         h += ["  return hipErrorInvalidValue;", "}", ""]
     for dtype, vec, w in ROWWISE:

@@ -27,6 +27,7 @@ def _gen(seed):
     (torch.float32, 64, 64), (torch.float32, 128, 320), (torch.float32, 1024, 512), (torch.float32, 32, 256),
     (torch.float32, 96, 768), (torch.float16, 64, 64), (torch.float16, 192, 128), (torch.float16, 512, 1024),
     (torch.float16, 64, 256), (torch.float16, 320, 768),
+    (torch.float32, 2048, 1024), (torch.float32, 4096, 3072),    # windowed cache-resident fp32 tiling
     (torch.float16, 8192, 2048),                    # one window of the windowed tile order
 ])
 def test_transpose_matches_oracle(ops, dtype, rows, cols):

@@ -30,7 +30,7 @@ def conflicts(word_addrs, words_per_lane, write=False):
     return worst
 
 
-@pytest.mark.parametrize("esize,tile,group", [(4, (32, 32), (1, 8)), (4, (32, 32), (2, 2)),
+@pytest.mark.parametrize("esize,tile,group", [(4, (32, 32), (1, 8)), (4, (32, 32), (2, 2)), (4, (32, 32), (2, 4)),
                                               (2, (64, 64), (1, 4)), (2, (64, 64), (1, 1))])
 def test_transpose_staging_is_bijective_and_conflict_free(esize, tile, group):
     sr, sc = tile[0] * group[0], tile[1] * group[1]
