@@ -25,13 +25,15 @@ MAX_GROUPS = 64
 
 
 def lds_a_layout(bm, chunks):
-    """A tile in 16-byte chunks: ``row*chunks + (chunk ^ ((row//2) % chunks))``.
+    """A tile in 16-byte chunks: ``row*chunks + (chunk ^ ((row // (16/chunks)) % chunks))``.
 
     Sixteen lanes that read the same chunk of sixteen consecutive rows (one quarter of a
-    ds_read_b128) land on sixteen different 16-byte slots of the 256-byte bank window,
-    and so do the sixteen lanes that write two whole rows."""
+    ds_read_b128) land on sixteen different 16-byte slots of the 256-byte bank window:
+    ``16/chunks`` consecutive rows fill the window once, and the key steps with every refill."""
+    assert 16 % chunks == 0
+
     def key(row):
-        return (row // 2) % chunks
+        return (row // (16 // chunks)) % chunks
 
     def forward(rc):
         row, ch = rc
@@ -106,6 +108,13 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
     B_ITERS = bk * bn // 8 // THREADS
     assert bm * bk // 8 % THREADS == 0 and bk * bn // 8 % THREADS == 0 and bk % 16 == 0
     assert WN >= 128, "the epilogue's staging rotation needs 32 eight-byte chunks per row"
+    # slot schedule of the main loop: a phase has TM*TN MFMA slots; even slots carry the TM+TN
+    # fragment loads, odd slots one memory->LDS instruction each, in the phase after the barrier
+    # (the first DMA_P3 of a k-tile) and in the phase that follows it (the rest)
+    SLOTS = TM * TN
+    assert TM + TN <= (SLOTS + 1) // 2 and bk == 64, "the four-phase slot schedule is laid out for 64-deep k-tiles"
+    DMA_P3 = min(A_ITERS + B_ITERS, SLOTS // 2)
+    assert A_ITERS + B_ITERS - DMA_P3 <= SLOTS // 2
 
     M, N, K = size("M"), size("N"), size("K")
     npm, npn, per_xcd, group_m = size("num_pid_m"), size("num_pid_n"), size("wg_per_xcd"), size("GM")
@@ -207,7 +216,7 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
 
     params = dict(
         banner=BANNER, BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
-        WM=WM, WN=WN, TM=TM, TN=TN, A_ITERS=A_ITERS, B_ITERS=B_ITERS, XCDS=XCDS, MAX_GROUPS=MAX_GROUPS,
+        WM=WM, WN=WN, TM=TM, TN=TN, A_ITERS=A_ITERS, B_ITERS=B_ITERS, DMA_P3=DMA_P3, XCDS=XCDS, MAX_GROUPS=MAX_GROUPS,
         pid_layout="OrderBy(Col(max(npm//GM,1),1), Col(min(npm,GM),npn)).TileBy([npm,npn]).inv(pid)",
         MAX_GM=max_group_m,
         xcd_layout=f"OrderBy(Col(nwg/{XCDS}, {XCDS})).TileBy([nwg/{XCDS}, {XCDS}])[Row(nwg/{XCDS}, {XCDS}).inv(wg)]",
