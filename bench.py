@@ -211,6 +211,17 @@ def main():
                 msv = timed(gv, steps=max(5, K // 5), warmup=max(2, W // 5))
                 kernels[f"next_gemm_f16_8192_{'t' if ta else 'n'}{'t' if tb else 'n'}"] = dict(
                     ms=msv, tflops=fl4 / msv / 1e9, frac_mfma=fl4 / msv / 1e9 / MFMA_F16_PEAK_TFLOPS)
+            ab, bb = a4.bfloat16(), b4.bfloat16()
+            cb = torch.empty_like(ab)
+
+            def gb():
+                runtime.call("lego_hip_gemm_bf16_ex", p(ab), p(bb), p(cb), n4, n4, n4, 0, 0, 0, stream)
+            msb = timed(gb, steps=max(5, K // 5), warmup=max(2, W // 5))
+            lib_msb = timed(lambda: torch.matmul(ab, bb, out=cb), steps=max(5, K // 5), warmup=max(2, W // 5))
+            kernels["next_gemm_bf16_8192"] = dict(ms=msb, tflops=fl4 / msb / 1e9,
+                                                  frac_mfma=fl4 / msb / 1e9 / MFMA_F16_PEAK_TFLOPS,
+                                                  vendor_library_tflops=fl4 / lib_msb / 1e9)
+            del ab, bb, cb
         del a4, b4, c4, ref
 
     # ---- C5: grouped fp16 GEMM, 8 problems -------------------------------------------------------------

@@ -70,6 +70,11 @@ int lego_hip_gemm_f16_act(const void* a, const void* b, void* c, int M, int N, i
  * to a K x M row-major buffer, trans_b != 0 means `b` points to an N x K row-major buffer. */
 int lego_hip_gemm_f16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                          int activation, void* stream);
+/* The same kernel for bfloat16 operands and result (fp32 accumulation).  The reference's matmul
+ * takes whatever 16-bit dtype its tensors have and stores fp16 (matmul_sympy.py:129-145, 203);
+ * here the result has the operands' type. */
+int lego_hip_gemm_bf16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
+                          int activation, void* stream);
 
 /* groups independent GEMMs in one launch.  a, b, c are HOST arrays of `groups` device
  * pointers; sizes3 is a HOST array of groups*3 ints (M, N, K per problem).  At most 64

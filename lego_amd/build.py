@@ -42,6 +42,7 @@ ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f32", True, 1
 ROWWISE_DEFAULT_WAVES = 4
 ROWWISE_MAX_N = 16384
 GEMM = dict(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8)
+GEMM_DTYPES = ("f16", "bf16")
 
 
 def generate():
@@ -58,10 +59,12 @@ def generate():
             units.append(unit)
             tmeta.setdefault(dtype, []).append(meta)
     units += [rowwise.emit(w, dtype, vec) for dtype, vec, w in ROWWISE]
-    for ta in (False, True):
-        for tb in (False, True):
-            g, mg = gemm.emit(**GEMM, trans_a=ta, trans_b=tb, with_grouped=not (ta or tb))
-            units.append(g)
+    for dtype in GEMM_DTYPES:
+        for ta in (False, True):
+            for tb in (False, True):
+                g, mg = gemm.emit(**GEMM, trans_a=ta, trans_b=tb, dtype=dtype,
+                                  with_grouped=dtype == "f16" and not (ta or tb))
+                units.append(g)
     lb, mlb = layernorm_bwd.emit()
     units.append(lb)
 
@@ -91,8 +94,8 @@ def generate():
           "hipError_t lego_layernorm_bwd_f16_launch(const void*, const void*, const void*, const float*, const float*, "
           "void*, void*, void*, float*, int, int, hipStream_t);",
           f"#define LEGO_LAYERNORM_BWD_MAX_N {mlb['MAX_N']}", ""]
-    h += [f"hipError_t lego_gemm_f16_{v}_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);"
-          for v in ("nn", "nt", "tn", "tt")]
+    h += [f"hipError_t lego_gemm_{d}_{v}_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);"
+          for d in GEMM_DTYPES for v in ("nn", "nt", "tn", "tt")]
     h += [
           "hipError_t lego_grouped_gemm_f16_launch(const void* const*, const void* const*, void* const*, "
           "const int*, int, hipStream_t);",

@@ -126,17 +126,32 @@ int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, con
                                              as_stream(stream)));
 }
 
-int lego_hip_gemm_f16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
-                         int activation, void* stream)
+namespace {
+typedef hipError_t (*gemm_launcher)(const void*, const void*, void*, int, int, int, int, hipStream_t);
+int gemm_ex(const gemm_launcher (&by_layout)[4], const void* a, const void* b, void* c, int M, int N, int K,
+            int trans_a, int trans_b, int activation, void* stream)
 {
   if (!usable(a) || !usable(b) || !usable(c)) return kInvalid;
   if (M <= 0 || N <= 0 || K <= 0 || M % LEGO_GEMM_BM || N % LEGO_GEMM_BN || K % LEGO_GEMM_BK) return kInvalid;
   if (activation != 0 && activation != 1) return kInvalid;
-  hipStream_t s = as_stream(stream);
-  if (!trans_a && !trans_b) return ok_or(lego_gemm_f16_nn_launch(a, b, c, M, N, K, activation, s));
-  if (!trans_a && trans_b) return ok_or(lego_gemm_f16_nt_launch(a, b, c, M, N, K, activation, s));
-  if (trans_a && !trans_b) return ok_or(lego_gemm_f16_tn_launch(a, b, c, M, N, K, activation, s));
-  return ok_or(lego_gemm_f16_tt_launch(a, b, c, M, N, K, activation, s));
+  return ok_or(by_layout[(trans_a ? 2 : 0) + (trans_b ? 1 : 0)](a, b, c, M, N, K, activation, as_stream(stream)));
+}
+}  // namespace
+
+int lego_hip_gemm_f16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
+                         int activation, void* stream)
+{
+  static const gemm_launcher by_layout[4] = {lego_gemm_f16_nn_launch, lego_gemm_f16_nt_launch,
+                                             lego_gemm_f16_tn_launch, lego_gemm_f16_tt_launch};
+  return gemm_ex(by_layout, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
+}
+
+int lego_hip_gemm_bf16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
+                          int activation, void* stream)
+{
+  static const gemm_launcher by_layout[4] = {lego_gemm_bf16_nn_launch, lego_gemm_bf16_nt_launch,
+                                             lego_gemm_bf16_tn_launch, lego_gemm_bf16_tt_launch};
+  return gemm_ex(by_layout, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
 }
 
 int lego_hip_gemm_f16_act(const void* a, const void* b, void* c, int M, int N, int K, int activation, void* stream)

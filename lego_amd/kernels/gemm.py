@@ -99,7 +99,10 @@ def xcd_remap(per, wg, xcds=XCDS):
     return OrderBy(Col(per, xcds)).TileBy([per, xcds])[j, x]
 
 
-def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, trans_b=False, with_grouped=True):
+def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, trans_b=False, with_grouped=True,
+         dtype="f16"):
+    elt = {"f16": "_Float16", "bf16": "__bf16"}[dtype]
+    assert not (with_grouped and dtype != "f16"), "the grouped kernel is built for fp16 only"
     WAVES_M, WAVES_N = waves
     THREADS = 64 * WAVES_M * WAVES_N
     WM, WN = bm // WAVES_M, bn // WAVES_N
@@ -215,7 +218,7 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
     chunk_params = dict(WAVES=WAVES, variant=variant, with_grouped=with_grouped, **operand("a"), **operand("b"))
 
     params = dict(
-        banner=BANNER, BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
+        banner=BANNER, elt=elt, dt=dtype, BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
         WM=WM, WN=WN, TM=TM, TN=TN, A_ITERS=A_ITERS, B_ITERS=B_ITERS, DMA_P3=DMA_P3, XCDS=XCDS, MAX_GROUPS=MAX_GROUPS,
         pid_layout="OrderBy(Col(max(npm//GM,1),1), Col(min(npm,GM),npn)).TileBy([npm,npn]).inv(pid)",
         MAX_GM=max_group_m,
@@ -239,5 +242,5 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
     )
     text = template("gemm.hip.j2").render(**params)
     meta = dict(BM=bm, BN=bn, BK=bk, MAX_GROUPS=MAX_GROUPS)
-    launchers = [f"lego_gemm_f16_{variant}_launch"] + (["lego_grouped_gemm_f16_launch"] if with_grouped else [])
-    return Emitted(f"gemm_f16_{variant}.hip", text, launchers), meta
+    launchers = [f"lego_gemm_{dtype}_{variant}_launch"] + (["lego_grouped_gemm_f16_launch"] if with_grouped else [])
+    return Emitted(f"gemm_{dtype}_{variant}.hip", text, launchers), meta

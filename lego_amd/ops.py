@@ -141,11 +141,14 @@ class LEGOLayerNorm(torch.autograd.Function):
 lego_layer_norm = LEGOLayerNorm.apply
 
 
+_GEMM_ENTRY = {torch.float16: "lego_hip_gemm_f16_ex", torch.bfloat16: "lego_hip_gemm_bf16_ex"}
+
+
 def _operand(t, name):
-    """``(storage tensor, transposed?)`` of a 2-D fp16 operand that is contiguous either as given
-    or as its transpose (the reference's TA/TB variants pass ``x.T`` views)."""
-    if not t.is_cuda or t.dtype != torch.float16 or t.dim() != 2:
-        raise ValueError(f"{name} must be a 2-D float16 GPU tensor")
+    """``(storage tensor, transposed?)`` of a 2-D fp16/bf16 operand that is contiguous either as
+    given or as its transpose (the reference's TA/TB variants pass ``x.T`` views)."""
+    if not t.is_cuda or t.dtype not in _GEMM_ENTRY or t.dim() != 2:
+        raise ValueError(f"{name} must be a 2-D float16 or bfloat16 GPU tensor")
     if t.is_contiguous():
         return t, 0
     if t.t().is_contiguous():
@@ -154,8 +157,8 @@ def _operand(t, name):
 
 
 def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "") -> torch.Tensor:
-    """``act(a @ b)`` for fp16 operands, each row-major or column-major (a ``.T`` view), fp32
-    accumulation, fp16 row-major result."""
+    """``act(a @ b)`` for fp16 (or bf16) operands, each row-major or column-major (a ``.T``
+    view), fp32 accumulation, row-major result of the operands' type."""
     if activation not in ("", "leaky_relu"):
         raise NotImplementedError(f"activation {activation!r} is not generated by this build")
     a_store, ta = _operand(a, "a")
@@ -164,8 +167,10 @@ def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "") -> torch.Tens
     K2, N = b.shape
     if K != K2:
         raise ValueError("Incompatible dimensions")
-    c = torch.empty((M, N), device=a.device, dtype=torch.float16)
-    runtime.call("lego_hip_gemm_f16_ex", _ptr(a_store), _ptr(b_store), _ptr(c), M, N, K, ta, tb,
+    if a.dtype != b.dtype:
+        raise ValueError("a and b must have the same dtype")
+    c = torch.empty((M, N), device=a.device, dtype=a.dtype)
+    runtime.call(_GEMM_ENTRY[a.dtype], _ptr(a_store), _ptr(b_store), _ptr(c), M, N, K, ta, tb,
                  1 if activation else 0, _stream())
     return c
 

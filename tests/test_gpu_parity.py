@@ -316,6 +316,40 @@ def test_gemm_transposed_integer_exact(ops):
             assert torch.equal(ops.matmul(ad, bd).cpu().double(), want)
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_gemm_bf16_matches_oracle(ops, ta, tb):
+    """bfloat16 operands and result: rel-err <= 1e-2 against fp32 accumulation (bf16 has 8
+    significand bits, so the rounding of the result alone is up to 2^-9 relative)."""
+    M, N, K = 512, 768, 320
+    print(f"gemm bf16 ta={ta} tb={tb} {M}x{N}x{K}", flush=True)
+    g = _gen(11)
+    a = (torch.randn(M, K, generator=g) / math.sqrt(K)).bfloat16()
+    b = (torch.randn(K, N, generator=g) / math.sqrt(K)).bfloat16()
+    want = ok.gemm(a, b)
+    ad = a.t().contiguous().cuda().t() if ta else a.cuda()
+    bd = b.t().contiguous().cuda().t() if tb else b.cuda()
+    got = ops.matmul(ad, bd)
+    assert got.dtype == torch.bfloat16
+    assert _rel_err(got.cpu(), want) <= 1e-2
+    # round-to-nearest-even of the fp32 accumulator: at most one bf16 spacing from the oracle
+    assert (got.cpu().float() - want.float()).abs().max().item() <= 2.0 ** -7
+
+
+def test_gemm_bf16_integer_exact(ops):
+    """Operands in {-1, 0, 1} and K = 256: every sum is an integer of magnitude <= 256, exact in
+    fp32 and in bf16."""
+    print("gemm bf16 integer exact", flush=True)
+    g = _gen(12)
+    a = torch.randint(-1, 2, (512, 256), generator=g).bfloat16()
+    b = torch.randint(-1, 2, (256, 768), generator=g).bfloat16()
+    want = a.double() @ b.double()
+    for ta in (False, True):
+        for tb in (False, True):
+            ad = a.t().contiguous().cuda().t() if ta else a.cuda()
+            bd = b.t().contiguous().cuda().t() if tb else b.cuda()
+            assert torch.equal(ops.matmul(ad, bd).cpu().double(), want)
+
+
 def test_gemm_leaky_relu_epilogue(ops):
     print("gemm leaky_relu", flush=True)
     g = _gen(8)
