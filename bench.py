@@ -25,7 +25,8 @@ import sys
 import time
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
-MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
+MFMA_FP8_PEAK_TFLOPS = 5000.0  # MI355X dense fp8 MFMA, published
 
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
 # what the same counters read for lego_hip_copy16 on 512 MiB (profiles/hbm_traffic_pmc.txt).
@@ -222,6 +223,22 @@ def main():
                                                   frac_mfma=fl4 / msb / 1e9 / MFMA_F16_PEAK_TFLOPS,
                                                   vendor_library_tflops=fl4 / lib_msb / 1e9)
             del ab, bb, cb
+            # 8-bit operands as the reference makes them: randn fp16 cast to float8_e5m2 (matmul_sympy.py:346-364)
+            g8 = gen(6)
+            a8 = torch.randn(n4, n4, generator=g8, dtype=torch.float16).to(torch.float8_e5m2).cuda()
+            b8 = torch.randn(n4, n4, generator=g8, dtype=torch.float16).to(torch.float8_e5m2).cuda()
+            c8 = torch.empty(n4, n4, dtype=torch.float16, device="cuda")
+
+            def g8f():
+                runtime.call("lego_hip_gemm_fp8_ex", p(a8), p(b8), p(c8), n4, n4, n4, 0, 0, 0, 1, stream)
+            g8f()
+            ref8 = a8[:256].float() @ b8.float()
+            rel8 = ((c8[:256].float() - ref8).norm() / ref8.norm()).item()
+            ms8 = timed(g8f, steps=max(5, K // 5), warmup=max(2, W // 5))
+            kernels["next_gemm_fp8_e5m2_8192"] = dict(ms=ms8, tflops=fl4 / ms8 / 1e9,
+                                                      frac_mfma=fl4 / ms8 / 1e9 / MFMA_FP8_PEAK_TFLOPS,
+                                                      rel_err_vs_fp32=rel8, note="peak = 5.0 PFLOP/s dense fp8")
+            del a8, b8, c8, ref8
         del a4, b4, c4, ref
 
     # ---- C5: grouped fp16 GEMM, 8 problems -------------------------------------------------------------
@@ -277,7 +294,8 @@ def main():
                      "kernel": "lego_transpose_f16_64x256_w128x8", "algorithmic_bytes_per_launch": bytes2},
         "cpu_baseline": cpu,
         "kernels": kernels,
-        "peaks": {"hbm_gbs": HBM_PEAK_GBS, "mfma_f16_tflops": MFMA_F16_PEAK_TFLOPS},
+        "peaks": {"hbm_gbs": HBM_PEAK_GBS, "mfma_f16_tflops": MFMA_F16_PEAK_TFLOPS,
+                  "mfma_fp8_tflops": MFMA_FP8_PEAK_TFLOPS},
     }
     print(json.dumps(line))
 

@@ -75,6 +75,12 @@ int lego_hip_gemm_f16_ex(const void* a, const void* b, void* c, int M, int N, in
  * here the result has the operands' type. */
 int lego_hip_gemm_bf16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                           int activation, void* stream);
+/* 8-bit floating-point operands, fp32 accumulation, fp16 result: the reference's fp8 path casts
+ * both operands to float8_e5m2 and stores fp16 (matmul_sympy.py:346-364, 203).  format 0 = OCP
+ * e4m3 (torch.float8_e4m3fn), 1 = OCP e5m2 (torch.float8_e5m2); a and b hold one byte per
+ * element; K must be a multiple of 128. */
+int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
+                         int activation, int format, void* stream);
 
 /* groups independent GEMMs in one launch.  a, b, c are HOST arrays of `groups` device
  * pointers; sizes3 is a HOST array of groups*3 ints (M, N, K per problem).  At most 64

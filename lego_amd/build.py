@@ -42,7 +42,8 @@ ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f32", True, 1
 ROWWISE_DEFAULT_WAVES = 4
 ROWWISE_MAX_N = 16384
 GEMM = dict(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8)
-GEMM_DTYPES = ("f16", "bf16")
+GEMM_DTYPES = ("f16", "bf16", "e4m3", "e5m2")
+GEMM_BK = {"f16": 64, "bf16": 64, "e4m3": 128, "e5m2": 128}   # 128 bytes of k per operand row in every case
 
 
 def generate():
@@ -62,9 +63,11 @@ def generate():
     for dtype in GEMM_DTYPES:
         for ta in (False, True):
             for tb in (False, True):
-                g, mg = gemm.emit(**GEMM, trans_a=ta, trans_b=tb, dtype=dtype,
+                g, m_ = gemm.emit(**dict(GEMM, bk=GEMM_BK[dtype]), trans_a=ta, trans_b=tb, dtype=dtype,
                                   with_grouped=dtype == "f16" and not (ta or tb))
                 units.append(g)
+                if dtype == "f16":
+                    mg = m_
     lb, mlb = layernorm_bwd.emit()
     units.append(lb)
 
@@ -100,6 +103,7 @@ def generate():
           "hipError_t lego_grouped_gemm_f16_launch(const void* const*, const void* const*, void* const*, "
           "const int*, int, hipStream_t);",
           f"#define LEGO_GEMM_BM {mg['BM']}", f"#define LEGO_GEMM_BN {mg['BN']}", f"#define LEGO_GEMM_BK {mg['BK']}",
+          f"#define LEGO_GEMM_BK_8BIT {GEMM_BK['e5m2']}",
           f"#define LEGO_GROUPED_MAX_GROUPS {mg['MAX_GROUPS']}", ""]
     GENERATED.mkdir(parents=True, exist_ok=True)
     header = GENERATED / "launchers.h"

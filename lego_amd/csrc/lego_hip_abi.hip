@@ -129,10 +129,10 @@ int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, con
 namespace {
 typedef hipError_t (*gemm_launcher)(const void*, const void*, void*, int, int, int, int, hipStream_t);
 int gemm_ex(const gemm_launcher (&by_layout)[4], const void* a, const void* b, void* c, int M, int N, int K,
-            int trans_a, int trans_b, int activation, void* stream)
+            int trans_a, int trans_b, int activation, void* stream, int bk = LEGO_GEMM_BK)
 {
   if (!usable(a) || !usable(b) || !usable(c)) return kInvalid;
-  if (M <= 0 || N <= 0 || K <= 0 || M % LEGO_GEMM_BM || N % LEGO_GEMM_BN || K % LEGO_GEMM_BK) return kInvalid;
+  if (M <= 0 || N <= 0 || K <= 0 || M % LEGO_GEMM_BM || N % LEGO_GEMM_BN || K % bk) return kInvalid;
   if (activation != 0 && activation != 1) return kInvalid;
   return ok_or(by_layout[(trans_a ? 2 : 0) + (trans_b ? 1 : 0)](a, b, c, M, N, K, activation, as_stream(stream)));
 }
@@ -152,6 +152,18 @@ int lego_hip_gemm_bf16_ex(const void* a, const void* b, void* c, int M, int N, i
   static const gemm_launcher by_layout[4] = {lego_gemm_bf16_nn_launch, lego_gemm_bf16_nt_launch,
                                              lego_gemm_bf16_tn_launch, lego_gemm_bf16_tt_launch};
   return gemm_ex(by_layout, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
+}
+
+int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
+                         int activation, int format, void* stream)
+{
+  static const gemm_launcher e4m3[4] = {lego_gemm_e4m3_nn_launch, lego_gemm_e4m3_nt_launch,
+                                        lego_gemm_e4m3_tn_launch, lego_gemm_e4m3_tt_launch};
+  static const gemm_launcher e5m2[4] = {lego_gemm_e5m2_nn_launch, lego_gemm_e5m2_nt_launch,
+                                        lego_gemm_e5m2_tn_launch, lego_gemm_e5m2_tt_launch};
+  if (format != 0 && format != 1) return kInvalid;
+  return gemm_ex(format == 0 ? e4m3 : e5m2, a, b, c, M, N, K, trans_a, trans_b, activation, stream,
+                 LEGO_GEMM_BK_8BIT);
 }
 
 int lego_hip_gemm_f16_act(const void* a, const void* b, void* c, int M, int N, int K, int activation, void* stream)

@@ -46,14 +46,16 @@ def lds_a_layout(bm, chunks):
     return OrderBy(GenP((bm, chunks), forward, backward)).TileBy([bm, chunks])
 
 
-def lds_b_layout(bk, bn):
-    """B tile in elements, rows of ``bn``: ``k*bn + (n ^ 32*(k % 4))``.
+def lds_b_layout(bk, bn, period=4):
+    """B tile in elements, rows of ``bn``: ``k*bn + (n ^ 32*(k % period))``.
 
-    A transposing read touches four consecutive k-rows, 64 bytes of each; rotating the
-    64-byte chunk index by ``k % 4`` puts the four rows on four different quarters of the
-    banks.  Bits 0-4 of ``n`` are untouched, so 16-byte stores and 8-byte reads stay whole."""
+    A transposing read of 2-byte elements touches four consecutive k-rows, 64 bytes of each;
+    rotating the 64-byte chunk index by ``k % 4`` puts the four rows on four different quarters
+    of the banks.  One of 1-byte elements touches eight k-rows, 32 bytes of each (32 elements
+    again): ``period = 8``.  Bits 0-4 of ``n`` are untouched, so 16-byte stores and 8-byte reads
+    stay whole."""
     def key(k):
-        return (k % 4) * 32
+        return (k % period) * 32
 
     def forward(kn):
         k, n = kn
@@ -101,21 +103,27 @@ def xcd_remap(per, wg, xcds=XCDS):
 
 def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, trans_b=False, with_grouped=True,
          dtype="f16"):
-    elt = {"f16": "_Float16", "bf16": "__bf16"}[dtype]
+    # element type, bytes per element, k-depth of one MFMA, result type; the 8-bit types are the
+    # OCP formats of v_mfma_f32_32x32x64_f8f6f4 (format code 0 = e4m3, 1 = e5m2)
+    elt, esize, mfma_k, out_elt = {"f16": ("_Float16", 2, 16, "_Float16"), "bf16": ("__bf16", 2, 16, "__bf16"),
+                                   "e4m3": ("unsigned char", 1, 64, "_Float16"),
+                                   "e5m2": ("unsigned char", 1, 64, "_Float16")}[dtype]
+    EPC = 16 // esize                      # elements per 16-byte chunk
     assert not (with_grouped and dtype != "f16"), "the grouped kernel is built for fp16 only"
     WAVES_M, WAVES_N = waves
     THREADS = 64 * WAVES_M * WAVES_N
     WM, WN = bm // WAVES_M, bn // WAVES_N
     TM, TN = WM // 32, WN // 32
-    A_ITERS = bm * bk // 8 // THREADS
-    B_ITERS = bk * bn // 8 // THREADS
-    assert bm * bk // 8 % THREADS == 0 and bk * bn // 8 % THREADS == 0 and bk % 16 == 0
+    A_ITERS = bm * bk // EPC // THREADS
+    B_ITERS = bk * bn // EPC // THREADS
+    assert bm * bk // EPC % THREADS == 0 and bk * bn // EPC % THREADS == 0 and bk % mfma_k == 0
+    NPH = bk // mfma_k                     # MFMA phases per k-tile
     assert WN >= 128, "the epilogue's staging rotation needs 32 eight-byte chunks per row"
     # slot schedule of the main loop: a phase has TM*TN MFMA slots; even slots carry the TM+TN
     # fragment loads, odd slots one memory->LDS instruction each, in the phase after the barrier
     # (the first DMA_P3 of a k-tile) and in the phase that follows it (the rest)
     SLOTS = TM * TN
-    assert TM + TN <= (SLOTS + 1) // 2 and bk == 64, "the four-phase slot schedule is laid out for 64-deep k-tiles"
+    assert TM + TN <= (SLOTS + 1) // 2 and NPH >= 2 and NPH % 2 == 0, "fragments are double buffered by phase parity"
     DMA_P3 = min(A_ITERS + B_ITERS, SLOTS // 2)
     assert A_ITERS + B_ITERS - DMA_P3 <= SLOTS // 2
 
@@ -141,9 +149,9 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
 
     wm_e, wn_e = OrderBy(Row(WAVES_M, WAVES_N)).TileBy([WAVES_M, WAVES_N]).inv(wave)
 
-    rng = {row: (0, bm), ch: (0, bk // 8), kr: (0, bk), i: (0, TM), j: (0, TN), r: (0, 16),
+    rng = {row: (0, bm), ch: (0, bk // EPC), kr: (0, bk), i: (0, TM), j: (0, TN), r: (0, 16),
            wm: (0, WAVES_M), wn: (0, WAVES_N), l32: (0, 32), lhi: (0, 2), l16: (0, 16),
-           lgrp: (0, 4), ks: (0, bk // 16), cr: (0, bm), cc: (0, bn), pid_m: (0, M / bm),
+           lgrp: (0, 4), ks: (0, NPH), cr: (0, bm), cc: (0, bn), pid_m: (0, M / bm),
            pid_n: (0, N / bn), k: (0, K / bk)}
 
     def chunk_walk(expr, n_iters):
@@ -193,21 +201,34 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
             return A_L[pid_m, k, row_e, kk_e] if role == "a" else B_L[k, pid_n, kk_e, row_e]
 
         if kmajor:
-            lds = lds_a_layout(rows, bk // 8)
+            lds = lds_a_layout(rows, bk // EPC)
             r_e, ch_e = (tidy(e, slot_rng) for e in lds.inv(slot))
-            full = tidy(glob(row, ch * 8), rng)
+            full = tidy(glob(row, ch * EPC), rng)
             placed = full.subs({row: r_e, ch: ch_e})
-            frag = ("*reinterpret_cast<const half8*>(%ss + (%s))"
-                    % (role, code(tidy(8 * lds[wave_off + l32, ks * 2 + lhi], rng))))
+            # a lane's mfma_k/2 k-values of row l32: one 16-byte chunk (2-byte elements) or two
+            n_ch = mfma_k // 2 // EPC
+            chunks = [code(tidy(EPC * lds[wave_off + l32, (ks * 2 + lhi) * n_ch + c], rng)) for c in range(n_ch)]
+            if esize == 2:
+                frag = "*reinterpret_cast<const half8*>(%ss + (%s))" % (role, chunks[0])
+            else:
+                frag = "read_k_fragment(%s)" % ", ".join("%ss + (%s)" % (role, c) for c in chunks)
         else:
-            lds = lds_b_layout(bk, rows)
-            kr_e, col_e = (tidy(e, slot_rng) for e in lds.inv(8 * slot))
-            full = tidy(glob(8 * ch, kr), rng)      # here `ch` counts 8-element chunks along the row
-            placed = full.subs({kr: kr_e, ch: tidy(col_e / 8, slot_rng)})
-            frag_k = [ks * 16 + (lgrp // 2) * 8 + h * 4 + l16 // 4 for h in (0, 1)]
-            frag_c = wave_off + (lgrp % 2) * 16 + 4 * (l16 % 4)
-            frag = ("read_b_fragment(%ss + (%s), %ss + (%s))"
-                    % (role, code(tidy(lds[frag_k[0], frag_c], rng)), role, code(tidy(lds[frag_k[1], frag_c], rng))))
+            lds = lds_b_layout(bk, rows, 4 if esize == 2 else 8)
+            kr_e, col_e = (tidy(e, slot_rng) for e in lds.inv(EPC * slot))
+            full = tidy(glob(EPC * ch, kr), rng)    # here `ch` counts 16-byte chunks along the row
+            placed = full.subs({kr: kr_e, ch: tidy(col_e / EPC, slot_rng)})
+            if esize == 2:
+                # a transposing read hands lane 16g+i four consecutive k of column i of group g's
+                # 16 columns; source lane s supplies k-row s/4 and columns 4*(s%4)..+3
+                frag_k = [ks * 16 + (lgrp // 2) * 8 + h * 4 + l16 // 4 for h in (0, 1)]
+                frag_c = wave_off + (lgrp % 2) * 16 + 4 * (l16 % 4)
+            else:
+                # 8-bit: eight consecutive k per read; source lane s supplies k-row s/2 and columns
+                # 8*(s%2)..+7 (even source lanes feed lanes 0-7 of the group, odd ones lanes 8-15)
+                frag_k = [ks * 64 + (lgrp // 2) * 32 + h * 8 + l16 // 2 for h in range(4)]
+                frag_c = wave_off + (lgrp % 2) * 16 + 8 * (l16 % 2)
+            frag = ("read_t_fragment(%s)"
+                    % ", ".join("%ss + (%s)" % (role, code(tidy(lds[fk, frag_c], rng))) for fk in frag_k))
         src0, step = chunk_walk(placed.subs({tile_id: 0, k: 0}), n_iters)
         return {f"{role}_src0": code(src0), f"{role}_src_step": code(step),
                 f"{role}_goff_base": code(full.subs({k: 0, row: 0, ch: 0, kr: 0})),
@@ -218,7 +239,8 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
     chunk_params = dict(WAVES=WAVES, variant=variant, with_grouped=with_grouped, **operand("a"), **operand("b"))
 
     params = dict(
-        banner=BANNER, elt=elt, dt=dtype, BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
+        banner=BANNER, elt=elt, out_elt=out_elt, ESIZE=esize, EPC=EPC, MFMA_K=mfma_k, NPH=NPH,
+        FMT={"e4m3": 0, "e5m2": 1}.get(dtype, 0), dt=dtype, BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
         WM=WM, WN=WN, TM=TM, TN=TN, A_ITERS=A_ITERS, B_ITERS=B_ITERS, DMA_P3=DMA_P3, XCDS=XCDS, MAX_GROUPS=MAX_GROUPS,
         pid_layout="OrderBy(Col(max(npm//GM,1),1), Col(min(npm,GM),npn)).TileBy([npm,npn]).inv(pid)",
         MAX_GM=max_group_m,

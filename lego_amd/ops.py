@@ -142,13 +142,14 @@ lego_layer_norm = LEGOLayerNorm.apply
 
 
 _GEMM_ENTRY = {torch.float16: "lego_hip_gemm_f16_ex", torch.bfloat16: "lego_hip_gemm_bf16_ex"}
+_FP8_FORMAT = {torch.float8_e4m3fn: 0, torch.float8_e5m2: 1}
 
 
 def _operand(t, name):
     """``(storage tensor, transposed?)`` of a 2-D fp16/bf16 operand that is contiguous either as
     given or as its transpose (the reference's TA/TB variants pass ``x.T`` views)."""
-    if not t.is_cuda or t.dtype not in _GEMM_ENTRY or t.dim() != 2:
-        raise ValueError(f"{name} must be a 2-D float16 or bfloat16 GPU tensor")
+    if not t.is_cuda or (t.dtype not in _GEMM_ENTRY and t.dtype not in _FP8_FORMAT) or t.dim() != 2:
+        raise ValueError(f"{name} must be a 2-D float16, bfloat16 or float8 GPU tensor")
     if t.is_contiguous():
         return t, 0
     if t.t().is_contiguous():
@@ -158,7 +159,8 @@ def _operand(t, name):
 
 def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "") -> torch.Tensor:
     """``act(a @ b)`` for fp16 (or bf16) operands, each row-major or column-major (a ``.T``
-    view), fp32 accumulation, row-major result of the operands' type."""
+    view), fp32 accumulation, row-major result of the operands' type.  float8_e5m2 (the
+    reference's fp8 path, matmul_sympy.py:346-364) and float8_e4m3fn operands give an fp16 result."""
     if activation not in ("", "leaky_relu"):
         raise NotImplementedError(f"activation {activation!r} is not generated by this build")
     a_store, ta = _operand(a, "a")
@@ -169,6 +171,11 @@ def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "") -> torch.Tens
         raise ValueError("Incompatible dimensions")
     if a.dtype != b.dtype:
         raise ValueError("a and b must have the same dtype")
+    if a.dtype in _FP8_FORMAT:
+        c = torch.empty((M, N), device=a.device, dtype=torch.float16)
+        runtime.call("lego_hip_gemm_fp8_ex", _ptr(a_store), _ptr(b_store), _ptr(c), M, N, K, ta, tb,
+                     1 if activation else 0, _FP8_FORMAT[a.dtype], _stream())
+        return c
     c = torch.empty((M, N), device=a.device, dtype=a.dtype)
     runtime.call(_GEMM_ENTRY[a.dtype], _ptr(a_store), _ptr(b_store), _ptr(c), M, N, K, ta, tb,
                  1 if activation else 0, _stream())

@@ -1,0 +1,121 @@
+"""CPU simulation of the GEMM kernels' data movement, from the generated text itself.
+
+The address expressions are taken out of the emitted HIP source and evaluated for every lane:
+where each memory->LDS instruction puts which bytes of the operand tile, and which bytes the
+fragment reads hand to each lane -- including the transposing LDS reads, simulated with the
+lane/element rule measured on gfx950:
+
+* ``ds_read_b64_tr_b16``: within a group of 16 lanes, lane ``i`` receives element ``i % 4`` of
+  source lanes ``i//4 + 4*j``, ``j = 0..3``;
+* ``ds_read_b64_tr_b8``: lane ``i`` receives byte ``i % 8`` of source lanes ``i//8 + 2*j``,
+  ``j = 0..7``.
+
+Expected: lane ``l`` of an MFMA operand holds row/column ``l % 32`` and the ``k``-values
+``(l // 32) * kk .. + kk - 1`` of the k-step, ``kk`` = 8 (16-bit) or 32 (8-bit), in order.
+"""
+import re
+
+import numpy as np
+import pytest
+
+from lego_amd.kernels import gemm
+
+
+def _c_eval(expr, env):
+    """Evaluate a printed C index expression (non-negative integers: ``/`` is floor division)."""
+    return eval(expr.replace("/", "//"), {"__builtins__": {}}, env)
+
+
+def _grab(text, pattern):
+    m = re.search(pattern, text)
+    assert m, pattern
+    return m.group(1)
+
+
+def _args(call):
+    """Top-level comma-separated arguments of ``name(arg, arg, ...)``."""
+    inner = call[call.index("(") + 1:call.rindex(")")]
+    out, depth, cur = [], 0, ""
+    for ch in inner:
+        if ch == "," and depth == 0:
+            out.append(cur)
+            cur = ""
+            continue
+        depth += ch == "("
+        depth -= ch == ")"
+        cur += ch
+    return out + [cur]
+
+
+@pytest.mark.parametrize("dtype,bk", [("f16", 64), ("e5m2", 128)])
+@pytest.mark.parametrize("variant", ["nn", "tt"])
+def test_fragments_receive_the_right_elements(dtype, bk, variant):
+    ta, tb = variant[0] == "t", variant[1] == "t"
+    unit, _ = gemm.emit(bk=bk, trans_a=ta, trans_b=tb, with_grouped=False, dtype=dtype)
+    text = unit.text
+    esize = 2 if dtype == "f16" else 1
+    epc = 16 // esize                       # elements per 16-byte chunk
+    kk = 8 if esize == 2 else 32            # k-values a lane holds per MFMA
+    M = N = 512
+    K = 2 * bk
+    sizes = dict(M=M, N=N, K=K)
+    for role, rows_total, kmajor in (("a", M, not ta), ("b", N, tb)):
+        src0 = _grab(text, r"const unsigned %s_src0 = \d \* \((.*)\);" % role)
+        step = _grab(text, r"%s_src_step = \d \* \((.*?)\)[,;]" % role)
+        iters = 256 * bk // epc // 256
+        # --- what the memory->LDS instructions leave in the LDS buffer: element ids of tile (0, 0)
+        lds = np.full(256 * bk, -1, dtype=np.int64)
+        for wave in range(4):
+            for lane in range(64):
+                base = _c_eval(src0, dict(sizes, wave=wave, lane=lane))
+                for it in range(iters):
+                    off = base + it * _c_eval(step, sizes)          # element offset inside the operand
+                    slot = (it * 4 + wave) * 64 + lane
+                    # element id = (row, k) of the tile: k-major storage has pitch K, the other pitch rows_total
+                    for e in range(epc):
+                        if kmajor:
+                            r_, k_ = divmod(off + e, K)
+                        else:
+                            k_, r_ = divmod(off + e, rows_total)
+                        assert 0 <= r_ < 256 and 0 <= k_ < bk
+                        assert lds[slot * epc + e] == -1
+                        lds[slot * epc + e] = r_ * bk + k_
+        assert (lds >= 0).all() and len(set(lds.tolist())) == 256 * bk    # the whole tile, once
+        # --- what the fragment reads hand to the lanes
+        frag = _grab(text, r"f%s\[BUF\]\[%s\] = (.*?); \}" % (role, "i" if role == "a" else "j"))
+        for ks in range(bk // (2 * kk)):
+            for sub in range(4):
+                for w in range(2):
+                    env0 = dict(ks=ks, i=sub, j=sub, wm=w, wn=w)
+                    want_row0 = w * 128 + sub * 32
+
+                    def addr(expr, lane):
+                        env = dict(env0, l32=lane % 32, lhi=lane // 32, l16=lane % 16, lgrp=lane // 16)
+                        return _c_eval(expr, env)
+
+                    got = np.zeros((64, kk), dtype=np.int64)
+                    if kmajor:
+                        ptrs = [frag[frag.index("+ (") + 2:frag.rindex(")")]] if esize == 2 else \
+                            [a[a.index("+ (") + 2:] for a in _args(frag)]
+                        for lane in range(64):
+                            vals = []
+                            for pexp in ptrs:
+                                p0 = addr(pexp, lane)
+                                assert p0 % epc == 0
+                                vals += lds[p0:p0 + epc].tolist()
+                            got[lane] = vals
+                    else:
+                        ptrs = [a[a.index("+ (") + 2:] for a in _args(frag)]
+                        per = 8 // esize                         # elements per 8-byte read
+                        for r, pexp in enumerate(ptrs):
+                            for lane in range(64):
+                                g, i_ = lane // 16, lane % 16
+                                for jj in range(per):
+                                    src = 16 * g + i_ // per + (16 // per) * jj
+                                    p0 = addr(pexp, src)
+                                    assert p0 % per == 0
+                                    got[lane, r * per + jj] = lds[p0 + i_ % per]
+                    for lane in range(64):
+                        row = want_row0 + lane % 32
+                        k0 = ks * 2 * kk + (lane // 32) * kk
+                        assert got[lane].tolist() == [row * bk + k0 + x for x in range(kk)], (role, ks, sub, w, lane)

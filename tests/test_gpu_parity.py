@@ -350,6 +350,43 @@ def test_gemm_bf16_integer_exact(ops):
             assert torch.equal(ops.matmul(ad, bd).cpu().double(), want)
 
 
+@pytest.mark.parametrize("fp8", [torch.float8_e5m2, torch.float8_e4m3fn])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_gemm_fp8_matches_oracle(ops, fp8, ta, tb):
+    """8-bit operands (the reference casts randn fp16 tensors to float8_e5m2, matmul_sympy.py:346-364):
+    products of two fp8 values are exact in fp32, so the result differs from the fp32 product of
+    the same fp8 values only by accumulation order and the fp16 rounding of the result."""
+    M, N, K = 512, 768, 384
+    print(f"gemm {fp8} ta={ta} tb={tb} {M}x{N}x{K}", flush=True)
+    g = _gen(13)
+    a = torch.randn(M, K, generator=g).half().to(fp8)
+    b = torch.randn(K, N, generator=g).half().to(fp8)
+    want = (a.float() @ b.float())
+    ad = a.t().contiguous().cuda().t() if ta else a.cuda()
+    bd = b.t().contiguous().cuda().t() if tb else b.cuda()
+    got = ops.matmul(ad, bd)
+    assert got.dtype == torch.float16 and got.shape == (M, N)
+    assert _rel_err(got.cpu(), want) <= 1e-2
+    assert (got.cpu().float() - want).abs().max().item() <= 0.125     # the reference's own atol
+
+
+def test_gemm_fp8_integer_exact(ops):
+    """Operands in {-2..2} (exact in both 8-bit formats), K = 256: every sum is an integer below
+    2048, exact in fp32 and fp16.  A lane/byte mix-up between the operands changes the integers."""
+    g = _gen(14)
+    a = torch.randint(-2, 3, (512, 256), generator=g).float()
+    b = torch.randint(-2, 3, (256, 768), generator=g).float()
+    want = a.double() @ b.double()
+    for fp8 in (torch.float8_e5m2, torch.float8_e4m3fn):
+        for ta in (False, True):
+            for tb in (False, True):
+                print(f"gemm {fp8} integer exact ta={ta} tb={tb}", flush=True)
+                a8, b8 = a.to(fp8), b.to(fp8)
+                ad = a8.t().contiguous().cuda().t() if ta else a8.cuda()
+                bd = b8.t().contiguous().cuda().t() if tb else b8.cuda()
+                assert torch.equal(ops.matmul(ad, bd).cpu().double(), want)
+
+
 def test_gemm_leaky_relu_epilogue(ops):
     print("gemm leaky_relu", flush=True)
     g = _gen(8)

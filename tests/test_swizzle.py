@@ -101,6 +101,28 @@ def test_gemm_lds_layouts_are_bijective_and_conflict_free():
             assert conflicts(addrs, 2) == 1
 
 
+def test_gemm_lds_layouts_8bit_are_bijective_and_conflict_free():
+    """One-byte operands: 128 k-values per tile, 32 per lane and MFMA."""
+    bm, bn, bk = 256, 256, 128
+    a = gemm.lds_a_layout(bm, bk // 16)
+    b = gemm.lds_b_layout(bk, bn, 8)
+    ta = np.array([[int(a.apply(r, c)) for c in range(bk // 16)] for r in range(bm)])
+    tb = np.array([[int(b.apply(k, n)) for n in range(bn)] for k in range(bk)])
+    assert sorted(ta.ravel().tolist()) == list(range(bm * bk // 16))
+    assert sorted(tb.ravel().tolist()) == list(range(bk * bn))
+    # A fragments: lane l reads chunks 4*ks + 2*(l/32) + {0, 1} of row l % 32, two ds_read_b128
+    for ks in range(2):
+        for c in range(2):
+            assert conflicts([4 * ta[l % 32, 4 * ks + 2 * (l // 32) + c] for l in range(64)], 4) == 1
+    # B fragments: transposing 8-byte reads, lane l -> k-row ks*64 + (l/32)*32 + 8*h + (l%16)/2,
+    # columns (l/16 % 2)*16 + 8*(l % 2) .. +7 (byte addresses -> words)
+    for ks in range(2):
+        for h in range(4):
+            addrs = [tb[ks * 64 + (l // 32) * 32 + 8 * h + (l % 16) // 2, ((l // 16) % 2) * 16 + 8 * (l % 2)] // 4
+                     for l in range(64)]
+            assert conflicts(addrs, 2) == 1
+
+
 def test_oracle_xor_swizzle_matches_product_family():
     blk = li.xor_swizzle(16, 64, unit=4, every=4, span=16)   # fp32 key of a 64-row tile, 16 vectors
     seen = set()
