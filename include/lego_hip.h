@@ -82,6 +82,14 @@ int lego_hip_gemm_bf16_ex(const void* a, const void* b, void* c, int M, int N, i
 int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                          int activation, int format, void* stream);
 
+/* Needleman-Wunsch score matrix (Rodinia's needle, the reference's anti-diagonal layout
+ * benchmark: benchmarks/cuda/nw_sympy.py:9-11, kernels needle_kernel_temp.cu:70-258, host
+ * needle.cu:165-260).  reference and matrix are (n+1) x (n+1) int32, row-major; row 0 and
+ * column 0 of matrix hold the borders (-i*penalty in Rodinia); on return
+ * matrix[i][j] = max(matrix[i-1][j-1] + reference[i][j], matrix[i][j-1] - penalty,
+ * matrix[i-1][j] - penalty) for i, j >= 1.  n a multiple of 64, at most 32768. */
+int lego_hip_nw_i32(const int* reference, int* matrix, int n, int penalty, void* stream);
+
 /* groups independent GEMMs in one launch.  a, b, c are HOST arrays of `groups` device
  * pointers; sizes3 is a HOST array of groups*3 ints (M, N, K per problem).  At most 64
  * groups; every M, N a multiple of 256 and K a multiple of 64.  Replaces

@@ -14,7 +14,7 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
-from .kernels import gemm, layernorm_bwd, rowwise, transpose
+from .kernels import gemm, layernorm_bwd, nw, rowwise, transpose
 from .kernels.common import BANNER, CSRC, GENERATED
 from .lego_hip import HIPCC_FLAGS, hipcc_path
 
@@ -70,6 +70,8 @@ def generate():
                     mg = m_
     lb, mlb = layernorm_bwd.emit()
     units.append(lb)
+    nwu, mnw = nw.emit()
+    units.append(nwu)
 
     h = [f"// {BANNER}", "#pragma once", "#include <hip/hip_runtime.h>", ""]
     for dtype, metas in tmeta.items():
@@ -105,6 +107,8 @@ def generate():
           f"#define LEGO_GEMM_BM {mg['BM']}", f"#define LEGO_GEMM_BN {mg['BN']}", f"#define LEGO_GEMM_BK {mg['BK']}",
           f"#define LEGO_GEMM_BK_8BIT {GEMM_BK['e5m2']}",
           f"#define LEGO_GROUPED_MAX_GROUPS {mg['MAX_GROUPS']}", ""]
+    h += ["hipError_t lego_nw_i32_launch(const int*, int*, int, int, hipStream_t);",
+          f"#define LEGO_NW_TILE {mnw['B']}", ""]
     GENERATED.mkdir(parents=True, exist_ok=True)
     header = GENERATED / "launchers.h"
     text = "\n".join(h)

@@ -176,6 +176,13 @@ int lego_hip_gemm_f16(const void* a, const void* b, void* c, int M, int N, int K
   return lego_hip_gemm_f16_ex(a, b, c, M, N, K, 0, 0, 0, stream);
 }
 
+int lego_hip_nw_i32(const int* reference, int* matrix, int n, int penalty, void* stream)
+{
+  if (!usable(reference) || !usable(matrix)) return kInvalid;
+  if (n <= 0 || n % LEGO_NW_TILE || n > 32768) return kInvalid;
+  return ok_or(lego_nw_i32_launch(reference, matrix, n, penalty, as_stream(stream)));
+}
+
 int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* const* c,
                               const int* sizes3, int groups, void* stream)
 {

@@ -1,0 +1,48 @@
+"""Generator of the Needleman-Wunsch kernel.
+
+The reference's contribution to this benchmark is one layout: the score tile that a block
+sweeps along its anti-diagonals is stored in anti-diagonal order,
+``OrderBy(GenP([n, n], antidiag)).TileBy((n, n))[i, j]``, so that the cells touched in one step
+are neighbours in shared memory (benchmarks/cuda/nw_sympy.py:9-11; the Rodinia kernel around it is
+benchmarks/cuda/nw/needle_kernel_temp.cu:70-160).  The recurrence is Rodinia's:
+``m[i][j] = max(m[i-1][j-1] + ref[i][j], m[i][j-1] - penalty, m[i-1][j] - penalty)``.
+
+Here a block is one 64-lane wavefront and a 64 x 64 tile: lane ``tx`` owns column ``tx`` and
+walks down it one anti-diagonal behind lane ``tx - 1``, so the west and north-west neighbours
+arrive by a lane shift and the north neighbour is the lane's own previous value -- the
+recurrence needs no shared memory and no barrier.  LDS holds two tiles in the reference's
+anti-diagonal layout: the substitution scores (read along anti-diagonals) and the results
+(written along anti-diagonals, then copied out row by row in 256-byte segments).  The
+offsets of the tiles of the ``(n+1) x (n+1)`` matrices are LEGO expressions as well.
+"""
+from __future__ import annotations
+
+import sympy as sp
+
+from ..lego import GenP, OrderBy, Row, antidiag
+from .common import BANNER, Emitted, code, idx, size, template, tidy
+
+B = 64
+
+
+def tile_layout(b=B):
+    """The reference's anti-diagonal layout of a ``b x b`` tile."""
+    return OrderBy(GenP([b, b], lambda x: antidiag(b, x), None)).TileBy((b, b))
+
+
+def emit():
+    cols = size("cols")                       # n + 1: row pitch of both matrices
+    by, bx, ty, tx = (idx(n) for n in ("by", "bx", "ty", "tx"))
+    # cell (ty, tx) of block (by, bx); row 0 and column 0 of the matrices are the borders
+    full = OrderBy(Row(cols, cols)).TileBy([cols, cols])
+    cell = tidy(full[by * B + 1 + ty, bx * B + 1 + tx], {ty: (0, B), tx: (0, B)})
+    i, j = sp.symbols("i j", integer=True, nonnegative=True)
+    lds = sp.simplify(tile_layout()[i, j])
+    params = dict(
+        banner=BANNER, B=B,
+        tile_layout=f"OrderBy(GenP([{B}, {B}], antidiag)).TileBy(({B}, {B}))[i, j]",
+        matrix_layout=f"OrderBy(Row(cols, cols)).TileBy([cols, cols])[{B}*by + 1 + ty, {B}*bx + 1 + tx]",
+        cell=code(cell), lds=code(lds),
+    )
+    text = template("nw.hip.j2").render(**params)
+    return Emitted("nw_i32.hip", text, ["lego_nw_i32_launch"]), dict(B=B)

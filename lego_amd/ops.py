@@ -204,3 +204,15 @@ def lego_group_gemm_fn(group_A, group_B):
     sz = (ctypes.c_int * (3 * groups))(*sizes)
     runtime.call("lego_hip_grouped_gemm_f16", pa, pb, pc, sz, groups, _stream())
     return group_C
+
+
+def needleman_wunsch(reference: torch.Tensor, matrix: torch.Tensor, penalty: int) -> torch.Tensor:
+    """Fills the ``(n+1) x (n+1)`` int32 score ``matrix`` in place (its first row and column are the
+    borders) from the substitution scores ``reference``; returns ``matrix``.  The reference's
+    benchmark is a whole program (benchmarks/cuda/nw/needle.cu:165-260) with no host callable."""
+    _check(reference, torch.int32, "reference")
+    _check(matrix, torch.int32, "matrix")
+    if reference.shape != matrix.shape or matrix.shape[0] != matrix.shape[1]:
+        raise ValueError("reference and matrix must be square and of the same shape")
+    runtime.call("lego_hip_nw_i32", _ptr(reference), _ptr(matrix), matrix.shape[0] - 1, int(penalty), _stream())
+    return matrix

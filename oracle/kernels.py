@@ -79,3 +79,20 @@ def grouped_pid(pid, num_pid_m, num_pid_n, group_m):
     first_m = group_id * group_m
     size_m = np.minimum(num_pid_m - first_m, group_m)
     return first_m + (pid % width) % size_m, (pid % width) // size_m
+
+
+def needleman_wunsch(reference, penalty):
+    """Rodinia's Needleman-Wunsch recurrence (benchmarks/cuda/nw/needle.cu:289-310, the reference's
+    own CPU check): borders ``-i*penalty``, then
+    ``m[i][j] = max(m[i-1][j-1] + ref[i][j], m[i][j-1] - penalty, m[i-1][j] - penalty)``,
+    evaluated one anti-diagonal at a time with numpy.  ``reference`` is ``(n+1) x (n+1)`` int32."""
+    ref = np.asarray(reference, dtype=np.int64)
+    n1 = ref.shape[0]
+    m = np.zeros((n1, n1), dtype=np.int64)
+    m[:, 0] = -np.arange(n1) * penalty
+    m[0, :] = -np.arange(n1) * penalty
+    for d in range(2, 2 * n1 - 1):                       # cells with i + j == d, i, j >= 1
+        i = np.arange(max(1, d - (n1 - 1)), min(d - 1, n1 - 1) + 1)
+        j = d - i
+        m[i, j] = np.maximum(np.maximum(m[i - 1, j - 1] + ref[i, j], m[i, j - 1] - penalty), m[i - 1, j] - penalty)
+    return m.astype(np.int32)

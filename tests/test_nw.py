@@ -1,0 +1,74 @@
+"""Needleman-Wunsch: the oracle is pinned on the CPU, the kernel against the oracle on the GPU."""
+import numpy as np
+import pytest
+import sympy as sp
+import torch
+
+from lego_amd.kernels import nw
+from oracle import kernels as ok
+
+
+def _loops(ref, penalty):
+    n1 = ref.shape[0]
+    m = [[0] * n1 for _ in range(n1)]
+    for i in range(n1):
+        m[i][0] = -i * penalty
+        m[0][i] = -i * penalty
+    for i in range(1, n1):
+        for j in range(1, n1):
+            m[i][j] = max(m[i - 1][j - 1] + int(ref[i, j]), m[i][j - 1] - penalty, m[i - 1][j] - penalty)
+    return np.array(m, dtype=np.int32)
+
+
+def test_oracle_matches_the_plain_double_loop():
+    rng = np.random.default_rng(0)
+    for n, penalty in ((7, 10), (16, 3), (33, 1)):
+        ref = rng.integers(-4, 12, size=(n + 1, n + 1)).astype(np.int32)
+        assert np.array_equal(ok.needleman_wunsch(ref, penalty), _loops(ref, penalty))
+
+
+def test_oracle_closed_form_without_substitution_scores():
+    """With zero scores a diagonal step is free and a gap costs ``penalty``: m[i][j] = -|i-j|*penalty."""
+    n = 40
+    got = ok.needleman_wunsch(np.zeros((n + 1, n + 1), dtype=np.int32), 7)
+    i, j = np.meshgrid(np.arange(n + 1), np.arange(n + 1), indexing="ij")
+    assert np.array_equal(got, -np.abs(i - j) * 7)
+
+
+def test_tile_layout_is_the_anti_diagonal_enumeration():
+    """The LDS layout of the kernel: a bijection of the 64 x 64 tile in which the cells of one
+    anti-diagonal are consecutive and ordered by row."""
+    b = nw.B
+    i, j = sp.symbols("i j", integer=True, nonnegative=True)
+    f = sp.lambdify([i, j], nw.tile_layout()[i, j], "math")
+    table = np.array([[int(f(a, c)) for c in range(b)] for a in range(b)])
+    assert sorted(table.ravel().tolist()) == list(range(b * b))
+    pos = 0
+    for d in range(2 * b - 1):
+        for a in range(max(0, d - b + 1), min(d, b - 1) + 1):
+            assert table[a, d - a] == pos
+            pos += 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,penalty", [(64, 10), (256, 10), (1024, 3), (2048, 10)])
+def test_gpu_matches_oracle(n, penalty):
+    from lego_amd import ops
+    print(f"needleman-wunsch n={n} penalty={penalty}", flush=True)
+    g = torch.Generator().manual_seed(20 + n)
+    ref = torch.randint(-4, 12, (n + 1, n + 1), generator=g, dtype=torch.int32)
+    want = torch.from_numpy(ok.needleman_wunsch(ref.numpy(), penalty))
+    m = torch.zeros((n + 1, n + 1), dtype=torch.int32)
+    m[:, 0] = -torch.arange(n + 1, dtype=torch.int32) * penalty
+    m[0, :] = -torch.arange(n + 1, dtype=torch.int32) * penalty
+    got = ops.needleman_wunsch(ref.cuda(), m.cuda(), penalty).cpu()
+    assert torch.equal(got, want)
+
+
+@pytest.mark.gpu
+def test_gpu_rejects_bad_sizes():
+    from lego_amd import ops
+    from lego_amd.runtime import LegoHipError
+    with pytest.raises(LegoHipError):
+        ops.needleman_wunsch(torch.zeros(101, 101, dtype=torch.int32, device="cuda"),
+                             torch.zeros(101, 101, dtype=torch.int32, device="cuda"), 10)
