@@ -82,6 +82,19 @@ int lego_hip_gemm_bf16_ex(const void* a, const void* b, void* c, int M, int N, i
 int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                          int activation, int format, void* stream);
 
+/* 3-D stencils on an n x n x n fp32 array (the reference's bricks benchmarks:
+ * benchmarks/cuda/bricks_f3d.py:8-22 with bricks/main_tmp.cu:24-104, and bricks_laplasian.py:8-33
+ * with bricks-laplace/main_tmp.cu:24-96).  bricks == 0: in and out are row-major; bricks != 0:
+ * they are stored as contiguous 8 x 8 x 8 bricks, bricks in row-major order.  Points closer
+ * than radius (1..3) to the boundary are not written.  n a multiple of 8, at most 1024.
+ *   f3d:        out = in*c[r][r][r] + sum over |di|,|dj|,|dk| <= r of in[+di,+dj,+dk] * c[di+r][dj+r][dk+r],
+ *               c an 8 x 8 x 8 array;
+ *   laplacian:  out = in*c[0] + sum over a = 1..r of c[a] * (the six neighbours at distance a),
+ *               c an array of r+1 floats. */
+int lego_hip_stencil_f3d_f32(const float* in, float* out, const float* c, int n, int radius, int bricks, void* stream);
+int lego_hip_stencil_laplacian_f32(const float* in, float* out, const float* c, int n, int radius, int bricks,
+                                   void* stream);
+
 /* Needleman-Wunsch score matrix (Rodinia's needle, the reference's anti-diagonal layout
  * benchmark: benchmarks/cuda/nw_sympy.py:9-11, kernels needle_kernel_temp.cu:70-258, host
  * needle.cu:165-260).  reference and matrix are (n+1) x (n+1) int32, row-major; row 0 and

@@ -14,7 +14,7 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
-from .kernels import gemm, layernorm_bwd, nw, rowwise, transpose
+from .kernels import gemm, layernorm_bwd, nw, rowwise, stencil, transpose
 from .kernels.common import BANNER, CSRC, GENERATED
 from .lego_hip import HIPCC_FLAGS, hipcc_path
 
@@ -72,6 +72,8 @@ def generate():
     units.append(lb)
     nwu, mnw = nw.emit()
     units.append(nwu)
+    stu, mst = stencil.emit()
+    units.append(stu)
 
     h = [f"// {BANNER}", "#pragma once", "#include <hip/hip_runtime.h>", ""]
     for dtype, metas in tmeta.items():
@@ -108,7 +110,9 @@ def generate():
           f"#define LEGO_GEMM_BK_8BIT {GEMM_BK['e5m2']}",
           f"#define LEGO_GROUPED_MAX_GROUPS {mg['MAX_GROUPS']}", ""]
     h += ["hipError_t lego_nw_i32_launch(const int*, int*, int, int, hipStream_t);",
-          f"#define LEGO_NW_TILE {mnw['B']}", ""]
+          f"#define LEGO_NW_TILE {mnw['B']}", "",
+          "hipError_t lego_stencil_f32_launch(const float*, float*, const float*, int, int, int, int, hipStream_t);",
+          f"#define LEGO_STENCIL_BRICK {mst['B']}", f"#define LEGO_STENCIL_MAX_RADIUS {mst['MAX_RADIUS']}", ""]
     GENERATED.mkdir(parents=True, exist_ok=True)
     header = GENERATED / "launchers.h"
     text = "\n".join(h)

@@ -176,6 +176,27 @@ int lego_hip_gemm_f16(const void* a, const void* b, void* c, int M, int N, int K
   return lego_hip_gemm_f16_ex(a, b, c, M, N, K, 0, 0, 0, stream);
 }
 
+namespace {
+int stencil(const float* in, float* out, const float* c, int n, int radius, int kind, int bricks, void* stream)
+{
+  if (!usable(in) || !usable(out) || c == nullptr || in == out) return kInvalid;
+  if (n <= 0 || n % LEGO_STENCIL_BRICK || n > 1024 || radius < 1 || radius > LEGO_STENCIL_MAX_RADIUS || 2 * radius >= n)
+    return kInvalid;
+  return ok_or(lego_stencil_f32_launch(in, out, c, n, radius, kind, bricks ? 1 : 0, as_stream(stream)));
+}
+}  // namespace
+
+int lego_hip_stencil_f3d_f32(const float* in, float* out, const float* c, int n, int radius, int bricks, void* stream)
+{
+  return stencil(in, out, c, n, radius, 0, bricks, stream);
+}
+
+int lego_hip_stencil_laplacian_f32(const float* in, float* out, const float* c, int n, int radius, int bricks,
+                                   void* stream)
+{
+  return stencil(in, out, c, n, radius, 1, bricks, stream);
+}
+
 int lego_hip_nw_i32(const int* reference, int* matrix, int n, int penalty, void* stream)
 {
   if (!usable(reference) || !usable(matrix)) return kInvalid;

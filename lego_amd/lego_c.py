@@ -38,10 +38,28 @@ class LEGOCCodePrinter(NegativeProductMixin, C99CodePrinter):
         return f"(({self._print(num)})/({self._print(den)}))"
 
     def _print_Pow(self, expr):
-        if expr.exp.is_Integer and 2 <= int(expr.exp) <= 4:
+        # small integer powers as products, as the reference prints them (`i*i`,
+        # benchmarks/cuda/nw/needle_kernel.cu:10)
+        if self._is_product_power(expr):
             base = self.parenthesize(expr.base, precedence(expr))
             return "*".join([base] * int(expr.exp))
         return super()._print_Pow(expr)
+
+    @staticmethod
+    def _is_product_power(expr):
+        return expr.is_Pow and expr.exp.is_Integer and 2 <= int(expr.exp) <= 4
+
+    def _print_Mod(self, expr):
+        # An operand that is printed as a product must be parenthesised even though sympy ranks
+        # a Pow above `%`: `Mod(w, n**2)` is `w % (n*n)`, not `w % n*n`.
+        prec = precedence(expr)
+        parts = []
+        for arg in expr.args:
+            text = self.parenthesize(arg, prec)
+            if self._is_product_power(arg):
+                text = f"({text})"
+            parts.append(text)
+        return " % ".join(parts)
 
     def _fold_minmax(self, args, op):
         out = self._print(args[0])

@@ -216,3 +216,32 @@ def needleman_wunsch(reference: torch.Tensor, matrix: torch.Tensor, penalty: int
         raise ValueError("reference and matrix must be square and of the same shape")
     runtime.call("lego_hip_nw_i32", _ptr(reference), _ptr(matrix), matrix.shape[0] - 1, int(penalty), _stream())
     return matrix
+
+
+def _stencil(entry, x, c, radius, bricks, out):
+    _check(x, torch.float32, "x", ndim=3)
+    _check(c, torch.float32, "c", ndim=c.dim())
+    n = x.shape[0]
+    if x.shape != (n, n, n):
+        raise ValueError("x must be a cube")
+    out = torch.zeros_like(x) if out is None else out
+    runtime.call(entry, _ptr(x), _ptr(out), _ptr(c), n, int(radius), 1 if bricks else 0, _stream())
+    return out
+
+
+def stencil_f3d(x, c, radius=1, bricks=False, out=None):
+    """Dense ``(2*radius+1)^3`` stencil with the ``8 x 8 x 8`` coefficient cube ``c``; ``x`` holds the
+    ``n^3`` points row-major, or brick by brick when ``bricks`` is set (``x.view(-1)`` is the
+    storage either way).  Boundary points keep the value of ``out`` (zeros by default, as the
+    reference program's ``cudaMemset``, benchmarks/cuda/bricks/main_tmp.cu:160-163)."""
+    if c.shape != (8, 8, 8):
+        raise ValueError("c must be 8 x 8 x 8")
+    return _stencil("lego_hip_stencil_f3d_f32", x, c, radius, bricks, out)
+
+
+def stencil_laplacian(x, c, radius=1, bricks=False, out=None):
+    """Star stencil ``c[0]*x + sum_a c[a]*(six neighbours at distance a)``; ``c`` has at least
+    ``radius + 1`` entries."""
+    if c.dim() != 1 or c.shape[0] < radius + 1:
+        raise ValueError("c must hold radius + 1 coefficients")
+    return _stencil("lego_hip_stencil_laplacian_f32", x, c, radius, bricks, out)

@@ -96,3 +96,47 @@ def needleman_wunsch(reference, penalty):
         j = d - i
         m[i, j] = np.maximum(np.maximum(m[i - 1, j - 1] + ref[i, j], m[i, j - 1] - penalty), m[i - 1, j] - penalty)
     return m.astype(np.int32)
+
+
+def bricks_order(n, b=8):
+    """Offsets of the ``n^3`` points in bricks storage (benchmarks/cuda/bricks_f3d.py:11-12):
+    ``OrderBy(Row(n/b, n/b, n/b), Row(b, b, b)).TileBy([n/b]*3, [b]*3)`` evaluated for every point,
+    as an int64 array of shape ``(n, n, n)`` indexed by global coordinates."""
+    nb = n // b
+    lay = li.tile_by(li.Order(li.row(nb, nb, nb), li.row(b, b, b)), [nb, nb, nb], [b, b, b])
+    off = lay.offsets()                                # indexed [bx, by, bz, i, j, k]
+    return np.ascontiguousarray(off.transpose(0, 3, 1, 4, 2, 5)).reshape(n, n, n)
+
+
+def stencil_f3d(x, c, radius):
+    """The dense stencil of benchmarks/cuda/bricks/main_tmp.cu:24-66 on a row-major ``n^3`` float32
+    array, in float64: the centre is weighted once on its own and once more inside the window
+    sum, boundary points are zero."""
+    x = np.asarray(x, dtype=np.float64)
+    c = np.asarray(c, dtype=np.float64)
+    n, r = x.shape[0], radius
+    out = np.zeros_like(x)
+    core = (slice(r, n - r),) * 3
+    acc = x[core] * c[r, r, r]
+    for di in range(-r, r + 1):
+        for dj in range(-r, r + 1):
+            for dk in range(-r, r + 1):
+                acc = acc + x[r + di:n - r + di, r + dj:n - r + dj, r + dk:n - r + dk] * c[di + r, dj + r, dk + r]
+    out[core] = acc
+    return out
+
+
+def stencil_laplacian(x, c, radius):
+    """The star stencil of benchmarks/cuda/bricks-laplace/main_tmp.cu:24-57, in float64."""
+    x = np.asarray(x, dtype=np.float64)
+    c = np.asarray(c, dtype=np.float64)
+    n, r = x.shape[0], radius
+    out = np.zeros_like(x)
+    core = (slice(r, n - r),) * 3
+    acc = x[core] * c[0]
+    for a in range(1, r + 1):
+        acc = acc + c[a] * (x[r + a:n - r + a, r:n - r, r:n - r] + x[r - a:n - r - a, r:n - r, r:n - r]
+                            + x[r:n - r, r + a:n - r + a, r:n - r] + x[r:n - r, r - a:n - r - a, r:n - r]
+                            + x[r:n - r, r:n - r, r + a:n - r + a] + x[r:n - r, r:n - r, r - a:n - r - a])
+    out[core] = acc
+    return out

@@ -98,3 +98,17 @@ def test_sympy_mod_product_defect_is_guarded():
         e = sp.Mod(c * sp.Mod(y, n), q)
         for v in range(0, 80, 3):
             assert int(e.subs(y, v)) == (c * (v % n)) % q
+
+
+def test_mod_by_a_power_is_parenthesised():
+    """Small integer powers are printed as products (as the reference does); as an operand of
+    ``%`` such a product needs parentheses that sympy's precedence table does not ask for."""
+    from lego_amd.lego_c import LEGOCCodePrinter
+    w, n = sp.symbols("w n", integer=True, positive=True)
+    for printer in (LEGOHipCodePrinter(), LEGOCCodePrinter()):
+        text = printer.doprint(sp.floor(sp.Mod(w, n**2) / n))
+        assert text == "((w % (n*n))/(n))"
+        for wv in range(0, 60, 7):
+            for nv in (2, 3, 5):
+                assert eval(text.replace("/", "//"), {}, {"w": wv, "n": nv}) == (wv % (nv * nv)) // nv
+        assert printer.doprint(sp.Mod(n**2, 7)) == "(n*n) % 7"
