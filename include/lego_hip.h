@@ -95,6 +95,12 @@ int lego_hip_stencil_f3d_f32(const float* in, float* out, const float* c, int n,
 int lego_hip_stencil_laplacian_f32(const float* in, float* out, const float* c, int n, int radius, int bricks,
                                    void* stream);
 
+/* LU decomposition without pivoting of an n x n fp32 row-major matrix, in place: on return the
+ * strict lower triangle holds L (unit diagonal implied) and the upper triangle holds U, as
+ * Rodinia's lud (the reference's thread-coarsening benchmark: benchmarks/cuda/lud.py:5-12,
+ * kernels lud/lud_kernel_temp.cu:14-352, host loop :358-390).  n a multiple of 64, at most 32768. */
+int lego_hip_lud_f32(float* m, int n, void* stream);
+
 /* Needleman-Wunsch score matrix (Rodinia's needle, the reference's anti-diagonal layout
  * benchmark: benchmarks/cuda/nw_sympy.py:9-11, kernels needle_kernel_temp.cu:70-258, host
  * needle.cu:165-260).  reference and matrix are (n+1) x (n+1) int32, row-major; row 0 and

@@ -14,7 +14,7 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
-from .kernels import gemm, layernorm_bwd, nw, rowwise, stencil, transpose
+from .kernels import gemm, layernorm_bwd, lud, nw, rowwise, stencil, transpose
 from .kernels.common import BANNER, CSRC, GENERATED
 from .lego_hip import HIPCC_FLAGS, hipcc_path
 
@@ -74,6 +74,8 @@ def generate():
     units.append(nwu)
     stu, mst = stencil.emit()
     units.append(stu)
+    luu, mlu = lud.emit()
+    units.append(luu)
 
     h = [f"// {BANNER}", "#pragma once", "#include <hip/hip_runtime.h>", ""]
     for dtype, metas in tmeta.items():
@@ -112,7 +114,8 @@ def generate():
     h += ["hipError_t lego_nw_i32_launch(const int*, int*, int, int, hipStream_t);",
           f"#define LEGO_NW_TILE {mnw['B']}", "",
           "hipError_t lego_stencil_f32_launch(const float*, float*, const float*, int, int, int, int, hipStream_t);",
-          f"#define LEGO_STENCIL_BRICK {mst['B']}", f"#define LEGO_STENCIL_MAX_RADIUS {mst['MAX_RADIUS']}", ""]
+          f"#define LEGO_STENCIL_BRICK {mst['B']}", f"#define LEGO_STENCIL_MAX_RADIUS {mst['MAX_RADIUS']}", "",
+          "hipError_t lego_lud_f32_launch(float*, int, hipStream_t);", f"#define LEGO_LUD_BLOCK {mlu['B']}", ""]
     GENERATED.mkdir(parents=True, exist_ok=True)
     header = GENERATED / "launchers.h"
     text = "\n".join(h)

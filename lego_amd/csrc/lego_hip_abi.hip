@@ -197,6 +197,13 @@ int lego_hip_stencil_laplacian_f32(const float* in, float* out, const float* c, 
   return stencil(in, out, c, n, radius, 1, bricks, stream);
 }
 
+int lego_hip_lud_f32(float* m, int n, void* stream)
+{
+  if (!usable(m)) return kInvalid;
+  if (n <= 0 || n % LEGO_LUD_BLOCK || n > 32768) return kInvalid;
+  return ok_or(lego_lud_f32_launch(m, n, as_stream(stream)));
+}
+
 int lego_hip_nw_i32(const int* reference, int* matrix, int n, int penalty, void* stream)
 {
   if (!usable(reference) || !usable(matrix)) return kInvalid;

@@ -245,3 +245,14 @@ def stencil_laplacian(x, c, radius=1, bricks=False, out=None):
     if c.dim() != 1 or c.shape[0] < radius + 1:
         raise ValueError("c must hold radius + 1 coefficients")
     return _stencil("lego_hip_stencil_laplacian_f32", x, c, radius, bricks, out)
+
+
+def lud(m: torch.Tensor) -> torch.Tensor:
+    """LU decomposition without pivoting, in place; returns ``m`` holding L below the diagonal
+    (unit diagonal implied) and U on and above it (benchmarks/cuda/lud/lud.cu: a whole program,
+    no host callable)."""
+    _check(m, torch.float32, "m")
+    if m.shape[0] != m.shape[1]:
+        raise ValueError("m must be square")
+    runtime.call("lego_hip_lud_f32", _ptr(m), m.shape[0], _stream())
+    return m

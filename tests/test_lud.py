@@ -1,0 +1,73 @@
+"""LU decomposition without pivoting: oracle pins on the CPU, parity on the GPU."""
+import numpy as np
+import pytest
+import scipy.linalg
+import torch
+
+from lego_amd.kernels import lud as lud_gen
+from oracle import kernels as ok
+
+
+def _dominant(n, seed):
+    """Strictly column-diagonally-dominant: partial pivoting never swaps, so a library LU with
+    pivoting is the decomposition without pivoting."""
+    rng = np.random.default_rng(seed)
+    a = rng.uniform(-1, 1, (n, n))
+    a[np.arange(n), np.arange(n)] = np.abs(a).sum(axis=0) + 1.0
+    return a
+
+
+def test_oracle_matches_scipy_on_dominant_matrices():
+    for n in (5, 64, 130):
+        a = _dominant(n, n)
+        p, l, u = scipy.linalg.lu(a)
+        assert np.array_equal(p, np.eye(n))
+        got = ok.lud(a)
+        assert np.allclose(np.tril(got, -1) + np.eye(n), l, atol=1e-12)
+        assert np.allclose(np.triu(got), u, atol=1e-10)
+
+
+def test_oracle_reconstructs_the_matrix():
+    a = _dominant(96, 7)
+    got = ok.lud(a)
+    l, u = np.tril(got, -1) + np.eye(96), np.triu(got)
+    assert np.allclose(l @ u, a, atol=1e-10)
+
+
+def test_coarsening_places_every_block_element_once():
+    """The reference's ``inv``: virtual thread (ii, jj, tid) -> (i, j, tid/T, tid%T); with
+    r = i*T + ty, c = j*T + tx the R*R*T*T virtual threads cover the block exactly once."""
+    import sympy as sp
+    ii, jj, tid = sp.symbols("ii jj tid", integer=True, nonnegative=True)
+    f = sp.lambdify([ii, jj, tid], lud_gen.coarsening(ii, jj, tid), "math")
+    T, R = lud_gen.T, lud_gen.R
+    seen = set()
+    for a in range(R):
+        for b in range(R):
+            for t in range(T * T):
+                i, j, ty, tx = (int(v) for v in f(a, b, t))
+                assert (i, j, ty, tx) == (a, b, t // T, t % T)
+                seen.add((i * T + ty, j * T + tx))
+    assert len(seen) == (R * T) ** 2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n", [64, 128, 512, 1024])
+def test_gpu_matches_oracle(n):
+    from lego_amd import ops
+    print(f"lud n={n}", flush=True)
+    a = _dominant(n, 100 + n).astype(np.float32)
+    want = ok.lud(a)
+    got = ops.lud(torch.from_numpy(a.copy()).cuda()).cpu().numpy().astype(np.float64)
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 2e-5 * scale
+    l, u = np.tril(got, -1) + np.eye(n), np.triu(got)
+    assert np.abs(l @ u - a).max() <= 1e-4 * scale
+
+
+@pytest.mark.gpu
+def test_gpu_rejects_bad_sizes():
+    from lego_amd import ops
+    from lego_amd.runtime import LegoHipError
+    with pytest.raises(LegoHipError):
+        ops.lud(torch.eye(100, device="cuda"))
