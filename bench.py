@@ -39,8 +39,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of configs to time (c1,c2,c3,c4,c5,extra); "
-                    "c2 is always timed; 'extra' adds LayerNorm backward and the transposed GEMM layouts")
+    ap.add_argument("--only", default="", help="comma list of configs to time (c1,c2,c3,c4,c5,extra,apps); "
+                    "c2 is always timed; 'extra' adds LayerNorm backward and the other GEMM layouts and element "
+                    "types, 'apps' the stencil, Needleman-Wunsch and LUD programs")
     ns = ap.parse_args()
     if ns.gpus != 1:
         print("bench.py: this build measures one MI355X; every configuration of the hot path is a "
@@ -263,6 +264,46 @@ def main():
         kernels["c5_grouped_gemm_f16"] = dict(ms=ms, tflops=fl5 / ms / 1e9, frac_mfma=fl5 / ms / 1e9 / MFMA_F16_PEAK_TFLOPS,
                                               flop=fl5, problems=dims, rel_err_vs_fp32=rel)
         del A, B, C
+
+    # ---- next rows: the reference's lego_c benchmark programs (stencils on bricks, Needleman-Wunsch, LUD) ----
+    if want("apps"):
+        n = 384
+        xs = (torch.rand(n, n, n, generator=gen(7)) * 2 - 1).to(dev)
+        ys = torch.zeros_like(xs)
+        cs = torch.rand(8, 8, 8, generator=gen(8)).to(dev)
+        cl = torch.tensor([-6.0, 1.0], device=dev)
+        for name, entry, cc in (("f3d", "lego_hip_stencil_f3d_f32", cs), ("laplacian", "lego_hip_stencil_laplacian_f32", cl)):
+            for bricks in (0, 1):
+                def st(entry=entry, cc=cc, bricks=bricks):
+                    runtime.call(entry, p(xs), p(ys), p(cc), n, 1, bricks, stream)
+                ms = timed(st, steps=max(5, K // 5), warmup=max(2, W // 5))
+                kernels[f"next_stencil_{name}_384_r1_{'bricks' if bricks else 'rowmajor'}"] = dict(
+                    ms=ms, gbs=2 * n ** 3 * 4 / ms / 1e6, bytes=2 * n ** 3 * 4)
+        del xs, ys
+        nn = 8192
+        refm = torch.randint(-4, 12, (nn + 1, nn + 1), generator=gen(9), dtype=torch.int32).to(dev)
+        mat = torch.zeros((nn + 1, nn + 1), dtype=torch.int32, device=dev)
+        border = -torch.arange(nn + 1, dtype=torch.int32, device=dev) * 10
+        mat[:, 0] = border
+        mat[0, :] = border
+
+        def nwf():
+            runtime.call("lego_hip_nw_i32", p(refm), p(mat), nn, 10, stream)
+        ms = timed(nwf, steps=3, warmup=1)
+        kernels["next_needleman_wunsch_8192"] = dict(ms=ms, gcells_per_s=nn * nn / ms / 1e6,
+                                                     note="255 launches, one per anti-diagonal of 64x64 tiles")
+        del refm, mat
+        nl = 4096
+        a0 = torch.rand(nl, nl, generator=gen(10)).to(dev) + nl * torch.eye(nl, device=dev)
+        wk = torch.empty_like(a0)
+
+        def luf():
+            wk.copy_(a0)
+            runtime.call("lego_hip_lud_f32", p(wk), nl, stream)
+        ms = timed(luf, steps=3, warmup=1) - timed(lambda: wk.copy_(a0), steps=3, warmup=1)
+        kernels["next_lud_f32_4096"] = dict(ms=ms, tflops=(2 / 3) * nl ** 3 / ms / 1e9,
+                                            note="time of a matrix copy subtracted; fp32 on the vector ALUs")
+        del a0, wk
 
     # ---- CPU baseline: the oracle on a bounded panel of the headline matrix ------------------------------
     cpu = None
