@@ -4,8 +4,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 Prints ONE JSON line.  A "step" is one launch of the headline workload, the fp16
-16384x16384 transpose through the LEGO tiled + XOR-swizzled staging layout (the second
-configuration of BASELINE.json); ``value`` is its effective HBM bandwidth with the input
+16384x16384 transpose through the LEGO tiled + XOR-swizzled staging layout (the configuration
+the headline metric is quoted on); ``value`` is its effective HBM bandwidth with the input
 already resident in device memory.  The other four configurations are timed in the same
 run with the same K and W and reported under ``kernels`` with their own roofline
 fractions.  ``cpu_baseline`` times the CPU oracle (index arrays through the two layouts +
