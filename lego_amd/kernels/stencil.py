@@ -19,7 +19,8 @@ so both storage orders give the stencil's result.
 
 A workgroup of 512 lanes is one brick; lane ``t`` is point ``Row(B, B, B).inv(t)`` of it, last
 coordinate fastest, so a wavefront touches 64 consecutive floats of a brick (bricks storage) or
-eight 32-byte runs (row-major storage).
+eight 32-byte runs (row-major storage).  The brick and a shell of ``radius`` points around it
+are staged in LDS once; the neighbours of a point are read from there.
 """
 from __future__ import annotations
 
@@ -47,6 +48,11 @@ def emit():
     rng = {x: (0, B * nb), y: (0, B * nb), z: (0, B * nb)}
     at = [code(tidy(L[x // B, y // B, z // B, x % B, y % B, z % B], rng)) for L in layouts(nb)]
     coeff = OrderBy(Row(8, 8, 8)).TileBy([8, 8, 8])[a, b_, c_]
+    # the shell cube in LDS: row-major H x H x H, H a compile-time constant of the kernel
+    H, h, hx, hy, hz = size("H"), idx("h"), idx("hx"), idx("hy"), idx("hz")
+    shell = OrderBy(Row(H, H, H)).TileBy([H, H, H])
+    halo_inv = [code(tidy(e, {h: (0, H * H * H)})) for e in shell.inv(h)]
+    halo_at = code(tidy(shell[hx, hy, hz], {hx: (0, H), hy: (0, H), hz: (0, H)}))
     params = dict(
         banner=BANNER, B=B, MAX_RADIUS=MAX_RADIUS,
         normal_layout=f"OrderBy(Row(N, N, N)).TileBy([N/{B}]*3, [{B}]*3)[x/{B}, y/{B}, z/{B}, x%{B}, y%{B}, z%{B}]",
@@ -54,6 +60,7 @@ def emit():
         brick=[code(tidy(e, {wg: (0, nb * nb * nb)})) for e in bxyz],
         point=[code(tidy(e, {t: (0, B * B * B)})) for e in ijk],
         at_normal=at[0], at_bricks=at[1], coeff=code(coeff),
+        halo_layout="OrderBy(Row(H, H, H)).TileBy([H, H, H])", halo_inv=halo_inv, halo_at=halo_at,
     )
     text = template("stencil.hip.j2").render(**params)
     return Emitted("stencil_f32.hip", text, ["lego_stencil_f32_launch"]), dict(B=B, MAX_RADIUS=MAX_RADIUS)
