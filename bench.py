@@ -110,7 +110,12 @@ def main():
     kernels["c2_transpose_f16_16384"] = dict(ms=ms2, gbs=gbs2, frac_hbm=gbs2 / HBM_PEAK_GBS,
                                              bytes=bytes2, parity="bit-exact")
     kernels["device_copy_512MiB"] = dict(ms=copy_ms, gbs=copy_gbs, frac_hbm=copy_gbs / HBM_PEAK_GBS,
-                                         note="torch copy_ of the same buffers: achievable ceiling")
+                                         note="torch copy_ of the same buffers")
+    stream_ms = timed(lambda: runtime.call("lego_hip_copy16_stream", p(x2), p(y2), ctypes.c_ulonglong(bytes2 // 2), stream))
+    kernels["device_copy_stream_512MiB"] = dict(
+        ms=stream_ms, gbs=bytes2 / stream_ms / 1e6, frac_hbm=bytes2 / stream_ms / 1e6 / HBM_PEAK_GBS,
+        note="non-temporal copy of the same buffers, one contiguous 16 KiB chunk per workgroup: what a kernel that "
+             "reads and writes every byte once reaches here")
     kernels["device_copy16_512MiB"] = dict(ms=copy16_ms, gbs=bytes2 / copy16_ms / 1e6,
                                            note="plain 16-byte-per-lane copy kernel of this library (counter calibration)")
 

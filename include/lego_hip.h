@@ -129,6 +129,11 @@ int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const 
  * No counterpart in the reference.  bench.py uses it as the same-run copy ceiling and the
  * profiles use it to calibrate the FETCH_SIZE / WRITE_SIZE counters at this access width. */
 int lego_hip_copy16(const void* in, void* out, unsigned long long bytes, void* stream);
+/* Streaming copy (no counterpart in the reference): non-temporal accesses, one contiguous 16 KiB
+ * chunk per workgroup -- the access pattern of the row kernels without their arithmetic, i.e.
+ * the bandwidth a kernel that reads and writes every byte once can reach on this part.
+ * bytes a multiple of 16384. */
+int lego_hip_copy16_stream(const void* in, void* out, unsigned long long bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -26,6 +26,19 @@ __global__ void __launch_bounds__(256) lego_copy16_kernel(const uint4* __restric
   for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = in[i];
 }
 
+// streaming copy: a workgroup owns one contiguous 16 KiB chunk, four non-temporal 16-byte loads
+// per lane in flight, then four non-temporal stores
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(256) lego_copy16_stream_kernel(const u32x4* __restrict__ in, u32x4* __restrict__ out)
+{
+  const size_t base = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x;
+  u32x4 v[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(in + base + u * 256);
+#pragma unroll
+  for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(v[u], out + base + u * 256);
+}
+
 }  // namespace
 
 extern "C" {
@@ -231,6 +244,14 @@ int lego_hip_copy16(const void* in, void* out, unsigned long long bytes, void* s
   const unsigned grid = static_cast<unsigned>(n / 256 < 256 * 32 ? (n + 255) / 256 : 256 * 32);
   hipLaunchKernelGGL(lego_copy16_kernel, dim3(grid), dim3(256), 0, as_stream(stream),
                      static_cast<const uint4*>(in), static_cast<uint4*>(out), n);
+  return ok_or(hipGetLastError());
+}
+
+int lego_hip_copy16_stream(const void* in, void* out, unsigned long long bytes, void* stream)
+{
+  if (!usable(in) || !usable(out) || bytes == 0 || bytes % 16384 || bytes / 16384 > 0x7fffffffull) return kInvalid;
+  hipLaunchKernelGGL(lego_copy16_stream_kernel, dim3(static_cast<unsigned>(bytes / 16384)), dim3(256), 0,
+                     as_stream(stream), static_cast<const u32x4*>(in), static_cast<u32x4*>(out));
   return ok_or(hipGetLastError());
 }
 
