@@ -42,12 +42,13 @@ def _check(t, dtype, name, ndim=2):
 def transpose(x: torch.Tensor) -> torch.Tensor:
     """``x.T`` materialised: the ``rows x cols`` row-major input copied into the
     column-major layout of the same logical matrix."""
-    if x.dtype not in (torch.float32, torch.float16):
-        raise ValueError("transpose supports float32 and float16")
+    if x.element_size() not in (2, 4):
+        raise ValueError("transpose moves 2-byte and 4-byte elements (float16, bfloat16, float32, int32, ...)")
     _check(x, x.dtype, "x")
     rows, cols = x.shape
     out = torch.empty((cols, rows), device=x.device, dtype=x.dtype)
-    entry = "lego_hip_transpose_f32" if x.dtype == torch.float32 else "lego_hip_transpose_f16"
+    # the kernels move bits: the entry point is chosen by element size
+    entry = "lego_hip_transpose_f32" if x.element_size() == 4 else "lego_hip_transpose_f16"
     runtime.call(entry, _ptr(x), _ptr(out), rows, cols, _stream())
     return out
 

@@ -65,6 +65,13 @@ def test_transpose_windowed_order_rectangular(ops):
     assert torch.equal(y, x.t())
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.int32, torch.int16])
+def test_transpose_moves_bits_of_any_2_or_4_byte_type(ops, dtype):
+    print(f"transpose {dtype}", flush=True)
+    x = torch.randint(-30000, 30000, (192, 256), generator=_gen(3)).to(dtype).cuda()
+    assert torch.equal(ops.transpose(x), x.t().contiguous())
+
+
 def test_transpose_rejects_bad_shapes(ops):
     from lego_amd.runtime import LegoHipError
     with pytest.raises(LegoHipError):
