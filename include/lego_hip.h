@@ -51,7 +51,7 @@ int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void
  * partial buffers become one fp32 workspace the caller provides (the reference's wrapper
  * allocates its buffers with torch as well): ask for its size first, any 16-byte aligned
  * device buffer of at least that many bytes will do; its contents need no initialisation.
- * N must be a multiple of 8 and at most 8192. */
+ * N must be a multiple of 8 and at most 16384. */
 int lego_hip_layernorm_bwd_workspace_bytes(int M, int N, unsigned long long* bytes);
 int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, const float* mean,
                                const float* rstd, void* dx, void* dw, void* db, void* workspace,

@@ -99,7 +99,7 @@ def generate():
           "// waves per row: one wave keeps short rows free of barriers, four waves keep the",
           "// register footprint of long rows small enough for full occupancy",
           f"inline int lego_rowwise_default_wpr(int n) {{ return n <= 2048 ? 1 : {ROWWISE_DEFAULT_WAVES}; }}", ""]
-    h += ["unsigned lego_layernorm_bwd_groups(int M);",
+    h += ["unsigned lego_layernorm_bwd_groups(int M, int N);",
           "hipError_t lego_layernorm_bwd_f16_launch(const void*, const void*, const void*, const float*, const float*, "
           "void*, void*, void*, float*, int, int, hipStream_t);",
           f"#define LEGO_LAYERNORM_BWD_MAX_N {mlb['MAX_N']}", ""]

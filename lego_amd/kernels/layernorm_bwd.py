@@ -15,9 +15,10 @@ from __future__ import annotations
 from ..lego import OrderBy, Row
 from .common import BANNER, Emitted, code, idx, size, template, tidy
 
-THREADS = 256
 MAX_GROUPS = 512      # workgroups of stage 1 = rows of the partial buffers
-VPTS = (1, 2, 4)      # 16-byte vectors per lane: rows of up to 8192 elements
+# (lanes per row, 16-byte vectors per lane): rows of up to 2048, 4096, 8192 and 16384 elements; the
+# longest rows take 512 lanes so that a lane's partial sums still fit its registers
+CONFIGS = ((256, 1), (256, 2), (256, 4), (512, 4))
 
 
 def emit():
@@ -28,17 +29,18 @@ def emit():
     X = OrderBy(Row(M, N)).TileBy([M, N / 8], [1, 8])
     P = OrderBy(Row(G, N)).TileBy([G, N / 8], [1, 8])
     params = dict(
-        banner=BANNER, THREADS=THREADS, WAVES=THREADS // 64, VPTS=list(VPTS), MAX_GROUPS=MAX_GROUPS,
+        banner=BANNER, CONFIGS=list(CONFIGS), MAX_GROUPS=MAX_GROUPS,
+        MAX_N_256=max(v for th, v in CONFIGS if th == 256) * 256 * 8,
         row_layout="OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])[step, wg]",
         x_layout="OrderBy(Row(M, N)).TileBy([M, N/8], [1, 8])[row, v, 0, :]",
         part_layout="OrderBy(Row(G, N)).TileBy([G, N/8], [1, 8])[wg, v, 0, :]",
         row=code(row_e),
         row_base=code(tidy(X[row, 0, 0, 0], {row: (0, M)})).replace("row", "static_cast<size_t>(row)"),
-        vec=code(it * THREADS + t),
+        vecs={th: code(it * th + t) for th in sorted({th for th, _ in CONFIGS})},
         vec_off=code(tidy(X[0, v, 0, 0], {v: (0, N / 8)})),
         stat_off=code(OrderBy(Row(M)).TileBy([M])[row,]),
         part_off=code(tidy(P[wg, v, 0, 0], {wg: (0, G), v: (0, N / 8)})).replace("wg", "static_cast<size_t>(wg)"),
     )
     text = template("layernorm_bwd.hip.j2").render(**params)
     return Emitted("layernorm_bwd_f16.hip", text, ["lego_layernorm_bwd_f16_launch"]), dict(
-        MAX_N=max(VPTS) * THREADS * 8, MAX_GROUPS=MAX_GROUPS)
+        MAX_N=max(th * v for th, v in CONFIGS) * 8, MAX_GROUPS=MAX_GROUPS)

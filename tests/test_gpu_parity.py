@@ -202,7 +202,8 @@ def test_layernorm_backward_reference_test(ops):
     assert torch.allclose(db.cpu().float(), bc.grad, atol=1e-2, rtol=2e-3)
 
 
-@pytest.mark.parametrize("M,N", [(1, 8), (3, 520), (700, 1024), (513, 2048), (64, 8192)])
+@pytest.mark.parametrize("M,N", [(1, 8), (3, 520), (700, 1024), (513, 2048), (64, 8192), (300, 8200), (129, 15872),
+                                 (40, 16384)])
 def test_layernorm_backward_matches_oracle(ops, M, N):
     print(f"layernorm backward {M}x{N}", flush=True)
     g = _gen(6)
