@@ -20,7 +20,13 @@ import torch
 from . import runtime
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    """The current stream's handle; asked for on every call, since the caller may switch streams."""
+    if _raw_stream is not None:      # a plain integer, without building a torch.cuda.Stream object
+        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
