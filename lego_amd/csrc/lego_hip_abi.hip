@@ -142,10 +142,11 @@ int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, con
 namespace {
 typedef hipError_t (*gemm_launcher)(const void*, const void*, void*, int, int, int, int, hipStream_t);
 int gemm_ex(const gemm_launcher (&by_layout)[4], const void* a, const void* b, void* c, int M, int N, int K,
-            int trans_a, int trans_b, int activation, void* stream, int bk = LEGO_GEMM_BK)
+            int trans_a, int trans_b, int activation, void* stream, int bk = LEGO_GEMM_BK, int chunk = 8)
 {
+  // M and N in whole 16-byte chunks (`chunk` elements), K in whole k-tiles; tiles may be ragged
   if (!usable(a) || !usable(b) || !usable(c)) return kInvalid;
-  if (M <= 0 || N <= 0 || K <= 0 || M % LEGO_GEMM_BM || N % LEGO_GEMM_BN || K % bk) return kInvalid;
+  if (M <= 0 || N <= 0 || K <= 0 || M % chunk || N % chunk || K % bk) return kInvalid;
   if (activation != 0 && activation != 1) return kInvalid;
   return ok_or(by_layout[(trans_a ? 2 : 0) + (trans_b ? 1 : 0)](a, b, c, M, N, K, activation, as_stream(stream)));
 }
@@ -176,7 +177,7 @@ int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, in
                                         lego_gemm_e5m2_tn_launch, lego_gemm_e5m2_tt_launch};
   if (format != 0 && format != 1) return kInvalid;
   return gemm_ex(format == 0 ? e4m3 : e5m2, a, b, c, M, N, K, trans_a, trans_b, activation, stream,
-                 LEGO_GEMM_BK_8BIT);
+                 LEGO_GEMM_BK_8BIT, 16);
 }
 
 int lego_hip_gemm_f16_act(const void* a, const void* b, void* c, int M, int N, int K, int activation, void* stream)
@@ -232,7 +233,7 @@ int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* 
   for (int g = 0; g < groups; ++g) {
     const int m = sizes3[3 * g], n = sizes3[3 * g + 1], k = sizes3[3 * g + 2];
     if (!usable(a[g]) || !usable(b[g]) || !usable(c[g])) return kInvalid;
-    if (m <= 0 || n <= 0 || k <= 0 || m % LEGO_GEMM_BM || n % LEGO_GEMM_BN || k % LEGO_GEMM_BK) return kInvalid;
+    if (m <= 0 || n <= 0 || k <= 0 || m % 8 || n % 8 || k % LEGO_GEMM_BK) return kInvalid;
   }
   return ok_or(lego_grouped_gemm_f16_launch(a, b, c, sizes3, groups, as_stream(stream)));
 }

@@ -230,7 +230,12 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
             frag = ("read_t_fragment(%s)"
                     % ", ".join("%ss + (%s)" % (role, code(tidy(lds[fk, frag_c], rng))) for fk in frag_k))
         src0, step = chunk_walk(placed.subs({tile_id: 0, k: 0}), n_iters)
+        # what bounds a chunk at a ragged edge: its row of the tile (k-major: the row changes with the
+        # instruction) or its first column (the other kind: the same for every instruction)
+        edge0, edge_step = chunk_walk(r_e if kmajor else col_e, n_iters)
+        assert kmajor or edge_step == 0
         return {f"{role}_src0": code(src0), f"{role}_src_step": code(step),
+                f"{role}_edge0": code(edge0), f"{role}_edge_step": code(edge_step),
                 f"{role}_goff_base": code(full.subs({k: 0, row: 0, ch: 0, kr: 0})),
                 f"{role}_kstep": code(sp.simplify(full.subs(k, k + 1) - full)),
                 f"{role}_frag_code": frag}

@@ -119,3 +119,42 @@ def test_fragments_receive_the_right_elements(dtype, bk, variant):
                         row = want_row0 + lane % 32
                         k0 = ks * 2 * kk + (lane // 32) * kk
                         assert got[lane].tolist() == [row * bk + k0 + x for x in range(kk)], (role, ks, sub, w, lane)
+
+
+@pytest.mark.parametrize("variant", ["nn", "nt", "tn", "tt"])
+def test_ragged_edges_skip_exactly_what_lies_outside(variant):
+    """The EDGE instantiation guards every memory->LDS chunk with ``edge0 + X*step < rem``.  For a
+    tile with ``rem`` valid rows (columns), replay the guards: every chunk that passes must lie
+    inside the operand, and every chunk with data of a valid row (column) must pass."""
+    ta, tb = variant[0] == "t", variant[1] == "t"
+    bk = 64
+    unit, _ = gemm.emit(bk=bk, trans_a=ta, trans_b=tb, with_grouped=False)
+    text = unit.text
+    K = 2 * bk
+    for role, kmajor in (("a", not ta), ("b", tb)):
+        src0 = _grab(text, r"const unsigned %s_src0 = \d \* \((.*)\);" % role)
+        step = _grab(text, r"%s_src_step = \d \* \((.*?)\)[,;]" % role)
+        edge0 = _grab(text, r"const unsigned a_edge0 = (.*), b_edge0 = .*;") if role == "a" else \
+            _grab(text, r"const unsigned a_edge0 = .*, b_edge0 = (.*);")
+        estep = int(_grab(text, r"%s_edge0 \+ \(.*?\) \* \((\d+)\) < %s_rem" % (role, "m" if role == "a" else "n")))
+        for rem in (8, 40, 128, 200, 248):
+            rows_total = rem                     # the operand ends where the tile's valid part ends
+            sizes = dict(M=rows_total, N=rows_total, K=K)
+            covered = set()
+            for wave in range(4):
+                for lane in range(64):
+                    base = _c_eval(src0, dict(sizes, wave=wave, lane=lane))
+                    e0 = _c_eval(edge0, dict(wave=wave, lane=lane))
+                    for it in range(8):
+                        if not e0 + it * estep < rem:
+                            continue
+                        off = base + it * _c_eval(step, sizes)
+                        # the chunk's eight elements must exist: pitch K (k-major) or rows_total
+                        for e in range(8):
+                            if kmajor:
+                                r_, k_ = divmod(off + e, K)
+                            else:
+                                k_, r_ = divmod(off + e, rows_total)
+                            assert 0 <= r_ < rem and 0 <= k_ < bk, (role, rem, wave, lane, it)
+                            covered.add((r_, k_))
+            assert covered == {(r, k) for r in range(rem) for k in range(bk)}, (role, rem)

@@ -284,6 +284,61 @@ def test_grouped_gemm_matches_oracle(ops):
         assert _rel_err(c.cpu(), w) <= 1e-2
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (8, 8, 64), (384, 640, 192), (1000, 264, 320), (256, 520, 64)])
+def test_gemm_ragged_tiles(ops, ta, tb, M, N, K):
+    """M and N in whole 16-byte chunks but not in whole 256 x 256 tiles (the reference's own
+    grouped test multiplies 128 x 128 x 128, grouped_gemm.py:316-350)."""
+    print(f"gemm ragged ta={ta} tb={tb} {M}x{N}x{K}", flush=True)
+    g = _gen(15)
+    a = (torch.randn(M, K, generator=g) / math.sqrt(K)).half()
+    b = (torch.randn(K, N, generator=g) / math.sqrt(K)).half()
+    want = ok.gemm(a, b)
+    ad = a.t().contiguous().cuda().t() if ta else a.cuda()
+    bd = b.t().contiguous().cuda().t() if tb else b.cuda()
+    # the result is carved out of a larger buffer filled with a sentinel: nothing outside M x N may change
+    buf = torch.full((M * N + 4096,), 7.0, dtype=torch.half, device="cuda")
+    from lego_amd import runtime
+    import ctypes
+    runtime.call("lego_hip_gemm_f16_ex", ctypes.c_void_p(ad.t().data_ptr() if ta else ad.data_ptr()),
+                 ctypes.c_void_p(bd.t().data_ptr() if tb else bd.data_ptr()), ctypes.c_void_p(buf.data_ptr()),
+                 M, N, K, int(ta), int(tb), 0, None)
+    torch.cuda.synchronize()
+    got = buf[:M * N].view(M, N).cpu()
+    assert _rel_err(got, want) <= 1e-2
+    assert (got.float() - want.float()).abs().max().item() <= 1e-2
+    assert (buf[M * N:] == 7.0).all()
+    assert torch.equal(ops.matmul(ad, bd).cpu(), got)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e5m2, torch.float8_e4m3fn])
+def test_gemm_ragged_tiles_other_element_types(ops, dtype):
+    M, N, K = 272, 528, 256
+    print(f"gemm ragged {dtype} {M}x{N}x{K}", flush=True)
+    g = _gen(17)
+    a = torch.randn(M, K, generator=g).half().to(dtype)
+    b = torch.randn(K, N, generator=g).half().to(dtype)
+    want = a.float() @ b.float()
+    for ta in (False, True):
+        for tb in (False, True):
+            ad = a.t().contiguous().cuda().t() if ta else a.cuda()
+            bd = b.t().contiguous().cuda().t() if tb else b.cuda()
+            got = ops.matmul(ad, bd).cpu().float()
+            assert _rel_err(got, want) <= 1e-2, (ta, tb)
+
+
+def test_grouped_gemm_reference_test_shapes(ops):
+    """The reference's own grouped test: 1024, 512, 256 and 128 cubed (grouped_gemm.py:316-350)."""
+    print("grouped gemm 1024/512/256/128 cubed", flush=True)
+    g = _gen(16)
+    A = [torch.rand(n, n, generator=g).half() for n in (1024, 512, 256, 128)]
+    B = [torch.rand(n, n, generator=g).half() for n in (1024, 512, 256, 128)]
+    want = ok.grouped_gemm(A, B)
+    got = ops.lego_group_gemm_fn([a.cuda() for a in A], [b.cuda() for b in B])
+    for c, w in zip(got, want):
+        assert _rel_err(c.cpu(), w) <= 1e-2
+
+
 def test_gemm_rejects_bad_shapes(ops):
     from lego_amd.runtime import LegoHipError
     with pytest.raises(LegoHipError):
