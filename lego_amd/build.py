@@ -59,6 +59,7 @@ def generate():
             unit.filename = meta["kernel"].replace("lego_", "", 1) + ".hip"
             units.append(unit)
             tmeta.setdefault(dtype, []).append(meta)
+    units.append(transpose.emit_any())
     units += [rowwise.emit(w, dtype, vec) for dtype, vec, w in ROWWISE]
     for dtype in GEMM_DTYPES:
         for ta in (False, True):
@@ -77,11 +78,12 @@ def generate():
     luu, mlu = lud.emit()
     units.append(luu)
 
-    h = [f"// {BANNER}", "#pragma once", "#include <hip/hip_runtime.h>", ""]
+    h = [f"// {BANNER}", "#pragma once", "#include <hip/hip_runtime.h>", "",
+         "hipError_t lego_transpose_any_launch(const void*, void*, int, int, int, hipStream_t);"]
     for dtype, metas in tmeta.items():
         for m in metas:
             h.append(f"hipError_t {m['kernel']}_launch(const void*, void*, int, int, hipStream_t);")
-        h += [f"// picks the first tiling that divides the shape; hipErrorInvalidValue if none does",
+        h += [f"// picks the first tiling that divides the shape, else the one-element-per-access kernel",
               f"inline hipError_t lego_transpose_{dtype}_dispatch(const void* in, void* out, int rows, int cols, "
               "hipStream_t stream) {"]
         for m in metas:
@@ -89,7 +91,7 @@ def generate():
                 f" && 2ull * rows * cols * {4 if dtype == 'f32' else 2} <= {m['max_bytes']}ull"
             h.append(f"  if (rows % {m['row_multiple']} == 0 && cols % {m['col_multiple']} == 0{fits}) "
                      f"return {m['kernel']}_launch(in, out, rows, cols, stream);")
-        h += ["  return hipErrorInvalidValue;", "}", ""]
+        h += [f"  return lego_transpose_any_launch(in, out, rows, cols, {4 if dtype == 'f32' else 2}, stream);", "}", ""]
     for dtype, vec, w in ROWWISE:
         tag = dtype if vec else dtype + "s"
         h += [f"hipError_t lego_softmax_{tag}_w{w}_launch(const void*, void*, int, int, hipStream_t);",

@@ -200,3 +200,20 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix=""):
     text = template("transpose.hip.j2").render(**params)
     return Emitted(f"transpose_{dtype}{suffix}.hip", text, [params["kernel"] + "_launch"]), dict(
         SR=SR, SC=SC, kernel=params["kernel"], row_multiple=SR * WI, col_multiple=SC * WJ)
+
+
+def emit_any():
+    """The one-element-per-access fallback for shapes that no vectorised tiling divides: the
+    reference's row-major source and column-major destination with run-time sizes."""
+    R, C = size("R"), size("C")
+    r, c, t = idx("r"), idx("c"), idx("t")
+    src = OrderBy(Row(R, C)).TileBy([R, C])
+    dst = OrderBy(Col(R, C)).TileBy([R, C])
+    ty_e, tx_e = OrderBy(Row(4, 64)).TileBy([4, 64]).inv(t)
+    rng = {r: (0, R), c: (0, C)}
+    params = dict(banner=BANNER, src_layout="OrderBy(Row(R, C)).TileBy([R, C])[r, c]",
+                  dst_layout="OrderBy(Col(R, C)).TileBy([R, C])[r, c]",
+                  src_off=code(tidy(src[r, c], rng)), dst_off=code(tidy(dst[r, c], rng)),
+                  tx=code(tidy(tx_e, {t: (0, 256)})), ty=code(tidy(ty_e, {t: (0, 256)})))
+    text = template("transpose_any.hip.j2").render(**params)
+    return Emitted("transpose_any.hip", text, ["lego_transpose_any_launch"])

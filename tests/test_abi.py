@@ -31,10 +31,11 @@ def test_library_exports_every_declared_symbol():
 
 def test_argument_validation_needs_no_gpu():
     lib = runtime.load_library()
-    # null pointers, misaligned pointers and shapes that do not divide the tiles are rejected on
+    # null pointers, misaligned pointers and sizes a kernel cannot take are rejected on
     # the host (hipErrorInvalidValue == 1) before anything touches a device
     assert lib.lego_hip_transpose_f32(None, None, 64, 64, None) == 1
-    assert lib.lego_hip_transpose_f16(ctypes.c_void_p(16), ctypes.c_void_p(4096), 100, 64, None) == 1
+    assert lib.lego_hip_transpose_f16(ctypes.c_void_p(16), ctypes.c_void_p(4096), 0, 64, None) == 1
+    assert lib.lego_hip_transpose_f16(ctypes.c_void_p(4096), ctypes.c_void_p(4096), 64, 64, None) == 1   # in place
     assert lib.lego_hip_transpose_f16(ctypes.c_void_p(8), ctypes.c_void_p(4096), 64, 64, None) == 1
     assert lib.lego_hip_softmax_f16(ctypes.c_void_p(16), ctypes.c_void_p(4096), 4, 0, None) == 1
     assert lib.lego_hip_softmax_f16_wpr(ctypes.c_void_p(16), ctypes.c_void_p(4096), 4, 12, 4, None) == 1

@@ -72,14 +72,35 @@ def test_transpose_moves_bits_of_any_2_or_4_byte_type(ops, dtype):
     assert torch.equal(ops.transpose(x), x.t().contiguous())
 
 
-def test_transpose_rejects_bad_shapes(ops):
+@pytest.mark.parametrize("dtype,rows,cols", [(torch.float32, 100, 64), (torch.float32, 32, 64), (torch.float32, 1, 1),
+                                             (torch.float16, 1823, 781), (torch.float16, 65, 4097), (torch.float32, 777, 3)])
+def test_transpose_of_any_shape(ops, dtype, rows, cols):
+    """Shapes no vectorised tiling divides go through the one-element-per-access kernel."""
+    print(f"transpose (any shape) {dtype} {rows}x{cols}", flush=True)
+    x = (torch.rand(rows, cols, generator=_gen(4)) * 2 - 1).to(dtype)
+    want = ok.transpose(x, 1, 1)
+    assert torch.equal(want, x.t().contiguous())
+    buf = torch.full((rows * cols + 1024,), 7.0, dtype=dtype, device="cuda")
+    out = buf[:rows * cols].view(cols, rows)
+    from lego_amd import runtime
+    import ctypes
+    xd = x.cuda()
+    runtime.call("lego_hip_transpose_f32" if dtype == torch.float32 else "lego_hip_transpose_f16",
+                 ctypes.c_void_p(xd.data_ptr()), ctypes.c_void_p(out.data_ptr()), rows, cols, None)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), want)
+    assert (buf[rows * cols:] == 7.0).all()       # nothing past the matrix was written
+
+
+def test_transpose_rejects_bad_arguments(ops):
     from lego_amd.runtime import LegoHipError
-    with pytest.raises(LegoHipError):
-        ops.transpose(torch.zeros(100, 64, device="cuda"))
-    with pytest.raises(LegoHipError):
-        ops.transpose(torch.zeros(32, 64, device="cuda"))     # 32 rows need the 32x256 tiling
     with pytest.raises(ValueError):
         ops.transpose(torch.zeros(64, 64, device="cuda").t())
+    with pytest.raises(LegoHipError):
+        x = torch.zeros(64, 64, device="cuda")
+        from lego_amd import runtime
+        import ctypes
+        runtime.call("lego_hip_transpose_f32", ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(x.data_ptr()), 64, 64, None)
 
 
 # ---- softmax / layernorm: max abs err <= 2e-3 ------------------------------------------------
