@@ -42,6 +42,8 @@ ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f32", True, 1
 ROWWISE_DEFAULT_WAVES = 4
 ROWWISE_MAX_N = 16384
 GEMM = dict(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8)
+GEMM_SMALL_TILE = 128
+GEMM_SMALL_DTYPES = ("f16", "bf16")     # a 128-byte row of 8-bit elements is too short for their [k][n] rotation
 GEMM_DTYPES = ("f16", "bf16", "e4m3", "e5m2")
 GEMM_BK = {"f16": 64, "bf16": 64, "e4m3": 128, "e5m2": 128}   # 128 bytes of k per operand row in every case
 
@@ -69,6 +71,12 @@ def generate():
                 units.append(g)
                 if dtype == "f16":
                     mg = m_
+                # the same kernel on 128x128 tiles, two workgroups per CU: for problems with too few
+                # 256x256 tiles to fill the chip
+                if dtype in GEMM_SMALL_DTYPES:
+                    gs, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK[dtype], bm=GEMM_SMALL_TILE, bn=GEMM_SMALL_TILE),
+                                      trans_a=ta, trans_b=tb, dtype=dtype, with_grouped=False)
+                    units.append(gs)
     lb, mlb = layernorm_bwd.emit()
     units.append(lb)
     nwu, mnw = nw.emit()
@@ -105,8 +113,9 @@ def generate():
           "hipError_t lego_layernorm_bwd_f16_launch(const void*, const void*, const void*, const float*, const float*, "
           "void*, void*, void*, float*, int, int, hipStream_t);",
           f"#define LEGO_LAYERNORM_BWD_MAX_N {mlb['MAX_N']}", ""]
-    h += [f"hipError_t lego_gemm_{d}_{v}_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);"
-          for d in GEMM_DTYPES for v in ("nn", "nt", "tn", "tt")]
+    h += [f"hipError_t lego_gemm_{d}_{v}{t}_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);"
+          for d in GEMM_DTYPES for v in ("nn", "nt", "tn", "tt")
+          for t in ("", f"_t{GEMM_SMALL_TILE}x{GEMM_SMALL_TILE}") if not t or d in GEMM_SMALL_DTYPES]
     h += [
           "hipError_t lego_grouped_gemm_f16_launch(const void* const*, const void* const*, void* const*, "
           "const int*, int, hipStream_t);",

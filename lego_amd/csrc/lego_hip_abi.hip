@@ -141,40 +141,56 @@ int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, con
 
 namespace {
 typedef hipError_t (*gemm_launcher)(const void*, const void*, void*, int, int, int, int, hipStream_t);
-int gemm_ex(const gemm_launcher (&by_layout)[4], const void* a, const void* b, void* c, int M, int N, int K,
+struct GemmKernels {
+  gemm_launcher big[4];     // 256 x 256 tiles, one workgroup per CU; index 2*trans_a + trans_b
+  gemm_launcher small[4];   // 128 x 128 tiles, two workgroups per CU (null: not built for this type)
+};
+// Fewer 256 x 256 tiles than this and the 128 x 128 kernel, with four times as many workgroups,
+// keeps more of the 256 CUs busy than its higher LDS traffic per flop costs.
+constexpr long kSmallTileBelow = 129;
+
+int gemm_ex(const GemmKernels& k, const void* a, const void* b, void* c, int M, int N, int K,
             int trans_a, int trans_b, int activation, void* stream, int bk = LEGO_GEMM_BK, int chunk = 8)
 {
   // M and N in whole 16-byte chunks (`chunk` elements), K in whole k-tiles; tiles may be ragged
   if (!usable(a) || !usable(b) || !usable(c)) return kInvalid;
   if (M <= 0 || N <= 0 || K <= 0 || M % chunk || N % chunk || K % bk) return kInvalid;
   if (activation != 0 && activation != 1) return kInvalid;
+  const long tiles = static_cast<long>((M + LEGO_GEMM_BM - 1) / LEGO_GEMM_BM) * ((N + LEGO_GEMM_BN - 1) / LEGO_GEMM_BN);
+  const gemm_launcher* by_layout = tiles < kSmallTileBelow && k.small[0] != nullptr ? k.small : k.big;
   return ok_or(by_layout[(trans_a ? 2 : 0) + (trans_b ? 1 : 0)](a, b, c, M, N, K, activation, as_stream(stream)));
 }
+
+#define LEGO_GEMM_KERNELS_BIG_ONLY(DT)                                                                 \
+  {{lego_gemm_##DT##_nn_launch, lego_gemm_##DT##_nt_launch, lego_gemm_##DT##_tn_launch,              \
+    lego_gemm_##DT##_tt_launch},                                                                       \
+   {nullptr, nullptr, nullptr, nullptr}}
+#define LEGO_GEMM_KERNELS(DT)                                                                          \
+  {{lego_gemm_##DT##_nn_launch, lego_gemm_##DT##_nt_launch, lego_gemm_##DT##_tn_launch,              \
+    lego_gemm_##DT##_tt_launch},                                                                       \
+   {lego_gemm_##DT##_nn_t128x128_launch, lego_gemm_##DT##_nt_t128x128_launch,                         \
+    lego_gemm_##DT##_tn_t128x128_launch, lego_gemm_##DT##_tt_t128x128_launch}}
 }  // namespace
 
 int lego_hip_gemm_f16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                          int activation, void* stream)
 {
-  static const gemm_launcher by_layout[4] = {lego_gemm_f16_nn_launch, lego_gemm_f16_nt_launch,
-                                             lego_gemm_f16_tn_launch, lego_gemm_f16_tt_launch};
-  return gemm_ex(by_layout, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
+  static const GemmKernels k = LEGO_GEMM_KERNELS(f16);
+  return gemm_ex(k, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
 }
 
 int lego_hip_gemm_bf16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                           int activation, void* stream)
 {
-  static const gemm_launcher by_layout[4] = {lego_gemm_bf16_nn_launch, lego_gemm_bf16_nt_launch,
-                                             lego_gemm_bf16_tn_launch, lego_gemm_bf16_tt_launch};
-  return gemm_ex(by_layout, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
+  static const GemmKernels k = LEGO_GEMM_KERNELS(bf16);
+  return gemm_ex(k, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
 }
 
 int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                          int activation, int format, void* stream)
 {
-  static const gemm_launcher e4m3[4] = {lego_gemm_e4m3_nn_launch, lego_gemm_e4m3_nt_launch,
-                                        lego_gemm_e4m3_tn_launch, lego_gemm_e4m3_tt_launch};
-  static const gemm_launcher e5m2[4] = {lego_gemm_e5m2_nn_launch, lego_gemm_e5m2_nt_launch,
-                                        lego_gemm_e5m2_tn_launch, lego_gemm_e5m2_tt_launch};
+  static const GemmKernels e4m3 = LEGO_GEMM_KERNELS_BIG_ONLY(e4m3);
+  static const GemmKernels e5m2 = LEGO_GEMM_KERNELS_BIG_ONLY(e5m2);
   if (format != 0 && format != 1) return kInvalid;
   return gemm_ex(format == 0 ? e4m3 : e5m2, a, b, c, M, N, K, trans_a, trans_b, activation, stream,
                  LEGO_GEMM_BK_8BIT, 16);

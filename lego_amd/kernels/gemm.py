@@ -69,19 +69,22 @@ def lds_b_layout(bk, bn, period=4):
 
 
 def lds_c_layout(rows, cols):
-    """A wave's block of C as fp16 in 8-byte chunks: ``row*(cols/4) + (chunk ^ (row % 32))``.
+    """A wave's block of C as fp16 in 8-byte chunks: ``row*(cols/4) + (chunk ^ (row % span))``,
+    ``span = min(32, cols/4)``.
 
     The accumulator layout makes 32 lanes store the same chunk of 32 consecutive rows; the
-    rotation spreads them over 32 different chunks of the 256-byte bank window."""
+    rotation spreads them over 32 different chunks of the 256-byte bank window (over 16, two
+    rows each, when a row has only 16 chunks)."""
     chunks = cols // 4
+    span = min(32, chunks)
 
     def forward(rc):
         row, ch = rc
-        return row * chunks + BitXor(sp.sympify(ch), sp.sympify(row % 32))
+        return row * chunks + BitXor(sp.sympify(ch), sp.sympify(row % span))
 
     def backward(flat):
         row, p = flat // chunks, flat % chunks
-        return (row, BitXor(sp.sympify(p), sp.sympify(row % 32)))
+        return (row, BitXor(sp.sympify(p), sp.sympify(row % span)))
 
     return OrderBy(GenP((rows, chunks), forward, backward)).TileBy([rows, chunks])
 
@@ -118,14 +121,28 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
     B_ITERS = bk * bn // EPC // THREADS
     assert bm * bk // EPC % THREADS == 0 and bk * bn // EPC % THREADS == 0 and bk % mfma_k == 0
     NPH = bk // mfma_k                     # MFMA phases per k-tile
-    assert WN >= 128, "the epilogue's staging rotation needs 32 eight-byte chunks per row"
-    # slot schedule of the main loop: a phase has TM*TN MFMA slots; even slots carry the TM+TN
-    # fragment loads, odd slots one memory->LDS instruction each, in the phase after the barrier
-    # (the first DMA_P3 of a k-tile) and in the phase that follows it (the rest)
-    SLOTS = TM * TN
-    assert TM + TN <= (SLOTS + 1) // 2 and NPH >= 2 and NPH % 2 == 0, "fragments are double buffered by phase parity"
-    DMA_P3 = min(A_ITERS + B_ITERS, SLOTS // 2)
-    assert A_ITERS + B_ITERS - DMA_P3 <= SLOTS // 2
+    assert WN >= 64 and WN % 32 == 0
+    # Slot schedule of the main loop.  A phase has TM*TN MFMA slots; the TM+TN fragment loads of the
+    # next phase and the memory->LDS instructions are spread evenly over them (for the 256x256
+    # tile: a fragment on every even slot, a copy on every odd one).  The copies of a k-tile go into
+    # the phase after the barrier (the first DMA_LAST) and the phase that follows it (the rest).
+    SLOTS, FRAGS, COPIES = TM * TN, TM + TN, A_ITERS + B_ITERS
+    assert NPH >= 2 and NPH % 2 == 0, "fragments are double buffered by phase parity"
+    DMA_LAST = min(COPIES, SLOTS // 2 if SLOTS >= 2 * FRAGS else SLOTS)
+    assert COPIES - DMA_LAST <= SLOTS
+
+    def spread(first, count):
+        """``count`` items ``first, first+1, ...`` on slots ``floor((q + 1/2) * SLOTS / count)``."""
+        out = [[] for _ in range(SLOTS)]
+        for q in range(count):
+            out[(2 * q + 1) * SLOTS // (2 * count)].append(first + q)
+        return out
+
+    load_slots = [[] for _ in range(SLOTS)]
+    for f in range(FRAGS):
+        load_slots[f * SLOTS // FRAGS].append(f)
+    dma_last, dma_first = spread(0, DMA_LAST), spread(DMA_LAST, COPIES - DMA_LAST)
+    none = [[] for _ in range(SLOTS)]
 
     M, N, K = size("M"), size("N"), size("K")
     npm, npn, per_xcd, group_m = size("num_pid_m"), size("num_pid_n"), size("wg_per_xcd"), size("GM")
@@ -241,12 +258,14 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
                 f"{role}_frag_code": frag}
 
     variant = ("t" if trans_a else "n") + ("t" if trans_b else "n")
-    chunk_params = dict(WAVES=WAVES, variant=variant, with_grouped=with_grouped, **operand("a"), **operand("b"))
+    tag = "" if (bm, bn) == (256, 256) else f"_t{bm}x{bn}"
+    chunk_params = dict(WAVES=WAVES, variant=variant, tag=tag, with_grouped=with_grouped, **operand("a"), **operand("b"))
 
     params = dict(
         banner=BANNER, elt=elt, out_elt=out_elt, ESIZE=esize, EPC=EPC, MFMA_K=mfma_k, NPH=NPH,
         FMT={"e4m3": 0, "e5m2": 1}.get(dtype, 0), dt=dtype, BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
-        WM=WM, WN=WN, TM=TM, TN=TN, A_ITERS=A_ITERS, B_ITERS=B_ITERS, DMA_P3=DMA_P3, XCDS=XCDS, MAX_GROUPS=MAX_GROUPS,
+        WM=WM, WN=WN, TM=TM, TN=TN, A_ITERS=A_ITERS, B_ITERS=B_ITERS, DMA_LAST=DMA_LAST,
+        load_slots=load_slots, dma_last=dma_last, dma_first=dma_first, dma_none=none, XCDS=XCDS, MAX_GROUPS=MAX_GROUPS,
         pid_layout="OrderBy(Col(max(npm//GM,1),1), Col(min(npm,GM),npn)).TileBy([npm,npn]).inv(pid)",
         MAX_GM=max_group_m,
         xcd_layout=f"OrderBy(Col(nwg/{XCDS}, {XCDS})).TileBy([nwg/{XCDS}, {XCDS}])[Row(nwg/{XCDS}, {XCDS}).inv(wg)]",
@@ -269,5 +288,5 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
     )
     text = template("gemm.hip.j2").render(**params)
     meta = dict(BM=bm, BN=bn, BK=bk, MAX_GROUPS=MAX_GROUPS)
-    launchers = [f"lego_gemm_{dtype}_{variant}_launch"] + (["lego_grouped_gemm_f16_launch"] if with_grouped else [])
-    return Emitted(f"gemm_{dtype}_{variant}.hip", text, launchers), meta
+    launchers = [f"lego_gemm_{dtype}_{variant}{tag}_launch"] + (["lego_grouped_gemm_f16_launch"] if with_grouped else [])
+    return Emitted(f"gemm_{dtype}_{variant}{tag}.hip", text, launchers), meta

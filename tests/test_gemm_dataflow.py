@@ -47,11 +47,11 @@ def _args(call):
     return out + [cur]
 
 
-@pytest.mark.parametrize("dtype,bk", [("f16", 64), ("e5m2", 128)])
+@pytest.mark.parametrize("dtype,bk,tile", [("f16", 64, 256), ("e5m2", 128, 256), ("f16", 64, 128)])
 @pytest.mark.parametrize("variant", ["nn", "tt"])
-def test_fragments_receive_the_right_elements(dtype, bk, variant):
+def test_fragments_receive_the_right_elements(dtype, bk, tile, variant):
     ta, tb = variant[0] == "t", variant[1] == "t"
-    unit, _ = gemm.emit(bk=bk, trans_a=ta, trans_b=tb, with_grouped=False, dtype=dtype)
+    unit, _ = gemm.emit(bm=tile, bn=tile, bk=bk, trans_a=ta, trans_b=tb, with_grouped=False, dtype=dtype)
     text = unit.text
     esize = 2 if dtype == "f16" else 1
     epc = 16 // esize                       # elements per 16-byte chunk
@@ -62,9 +62,9 @@ def test_fragments_receive_the_right_elements(dtype, bk, variant):
     for role, rows_total, kmajor in (("a", M, not ta), ("b", N, tb)):
         src0 = _grab(text, r"const unsigned %s_src0 = \d \* \((.*)\);" % role)
         step = _grab(text, r"%s_src_step = \d \* \((.*?)\)[,;]" % role)
-        iters = 256 * bk // epc // 256
+        iters = tile * bk // epc // 256
         # --- what the memory->LDS instructions leave in the LDS buffer: element ids of tile (0, 0)
-        lds = np.full(256 * bk, -1, dtype=np.int64)
+        lds = np.full(tile * bk, -1, dtype=np.int64)
         for wave in range(4):
             for lane in range(64):
                 base = _c_eval(src0, dict(sizes, wave=wave, lane=lane))
@@ -77,17 +77,17 @@ def test_fragments_receive_the_right_elements(dtype, bk, variant):
                             r_, k_ = divmod(off + e, K)
                         else:
                             k_, r_ = divmod(off + e, rows_total)
-                        assert 0 <= r_ < 256 and 0 <= k_ < bk
+                        assert 0 <= r_ < tile and 0 <= k_ < bk
                         assert lds[slot * epc + e] == -1
                         lds[slot * epc + e] = r_ * bk + k_
-        assert (lds >= 0).all() and len(set(lds.tolist())) == 256 * bk    # the whole tile, once
+        assert (lds >= 0).all() and len(set(lds.tolist())) == tile * bk    # the whole tile, once
         # --- what the fragment reads hand to the lanes
         frag = _grab(text, r"f%s\[BUF\]\[%s\] = (.*?); \}" % (role, "i" if role == "a" else "j"))
         for ks in range(bk // (2 * kk)):
-            for sub in range(4):
+            for sub in range(tile // 64):
                 for w in range(2):
                     env0 = dict(ks=ks, i=sub, j=sub, wm=w, wn=w)
-                    want_row0 = w * 128 + sub * 32
+                    want_row0 = w * (tile // 2) + sub * 32
 
                     def addr(expr, lane):
                         env = dict(env0, l32=lane % 32, lhi=lane // 32, l16=lane % 16, lgrp=lane // 16)
@@ -121,14 +121,15 @@ def test_fragments_receive_the_right_elements(dtype, bk, variant):
                         assert got[lane].tolist() == [row * bk + k0 + x for x in range(kk)], (role, ks, sub, w, lane)
 
 
+@pytest.mark.parametrize("tile", [256, 128])
 @pytest.mark.parametrize("variant", ["nn", "nt", "tn", "tt"])
-def test_ragged_edges_skip_exactly_what_lies_outside(variant):
+def test_ragged_edges_skip_exactly_what_lies_outside(variant, tile):
     """The EDGE instantiation guards every memory->LDS chunk with ``edge0 + X*step < rem``.  For a
     tile with ``rem`` valid rows (columns), replay the guards: every chunk that passes must lie
     inside the operand, and every chunk with data of a valid row (column) must pass."""
     ta, tb = variant[0] == "t", variant[1] == "t"
     bk = 64
-    unit, _ = gemm.emit(bk=bk, trans_a=ta, trans_b=tb, with_grouped=False)
+    unit, _ = gemm.emit(bm=tile, bn=tile, bk=bk, trans_a=ta, trans_b=tb, with_grouped=False)
     text = unit.text
     K = 2 * bk
     for role, kmajor in (("a", not ta), ("b", tb)):
@@ -137,7 +138,7 @@ def test_ragged_edges_skip_exactly_what_lies_outside(variant):
         edge0 = _grab(text, r"const unsigned a_edge0 = (.*), b_edge0 = .*;") if role == "a" else \
             _grab(text, r"const unsigned a_edge0 = .*, b_edge0 = (.*);")
         estep = int(_grab(text, r"%s_edge0 \+ \(.*?\) \* \((\d+)\) < %s_rem" % (role, "m" if role == "a" else "n")))
-        for rem in (8, 40, 128, 200, 248):
+        for rem in (r for r in (8, 40, 120, 128, 200, 248) if r <= tile):
             rows_total = rem                     # the operand ends where the tile's valid part ends
             sizes = dict(M=rows_total, N=rows_total, K=K)
             covered = set()
@@ -145,7 +146,7 @@ def test_ragged_edges_skip_exactly_what_lies_outside(variant):
                 for lane in range(64):
                     base = _c_eval(src0, dict(sizes, wave=wave, lane=lane))
                     e0 = _c_eval(edge0, dict(wave=wave, lane=lane))
-                    for it in range(8):
+                    for it in range(tile * bk // 8 // 256):
                         if not e0 + it * estep < rem:
                             continue
                         off = base + it * _c_eval(step, sizes)

@@ -348,6 +348,32 @@ def test_gemm_ragged_tiles_other_element_types(ops, dtype):
             assert _rel_err(got, want) <= 1e-2, (ta, tb)
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("M,N,K", [(3072, 3072, 128), (3080, 3000, 64)])
+def test_gemm_many_tiles(ops, ta, tb, M, N, K):
+    """More than 128 tiles of 256 x 256: the one-workgroup-per-CU kernel (smaller problems take
+    the 128 x 128 tiles), whole and ragged."""
+    print(f"gemm many tiles ta={ta} tb={tb} {M}x{N}x{K}", flush=True)
+    g = _gen(18)
+    a = (torch.randn(M, K, generator=g) / math.sqrt(K)).half()
+    b = (torch.randn(K, N, generator=g) / math.sqrt(K)).half()
+    want = ok.gemm(a, b)
+    ad = a.t().contiguous().cuda().t() if ta else a.cuda()
+    bd = b.t().contiguous().cuda().t() if tb else b.cuda()
+    got = ops.matmul(ad, bd).cpu()
+    assert _rel_err(got, want) <= 1e-2
+    assert (got.float() - want.float()).abs().max().item() <= 1e-2
+
+
+def test_gemm_bf16_many_tiles(ops):
+    print("gemm bf16 many tiles", flush=True)
+    g = _gen(19)
+    a = (torch.randn(3072, 128, generator=g) / math.sqrt(128)).bfloat16()
+    b = (torch.randn(128, 3328, generator=g) / math.sqrt(128)).bfloat16()
+    got = ops.matmul(a.cuda(), b.cuda()).cpu()
+    assert _rel_err(got, ok.gemm(a, b)) <= 1e-2
+
+
 def test_grouped_gemm_reference_test_shapes(ops):
     """The reference's own grouped test: 1024, 512, 256 and 128 cubed (grouped_gemm.py:316-350)."""
     print("grouped gemm 1024/512/256/128 cubed", flush=True)
