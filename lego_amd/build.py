@@ -75,7 +75,8 @@ def generate():
                 # 256x256 tiles to fill the chip
                 if dtype in GEMM_SMALL_DTYPES:
                     gs, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK[dtype], bm=GEMM_SMALL_TILE, bn=GEMM_SMALL_TILE),
-                                      trans_a=ta, trans_b=tb, dtype=dtype, with_grouped=False)
+                                      trans_a=ta, trans_b=tb, dtype=dtype,
+                                      with_grouped=dtype == "f16" and not (ta or tb))
                     units.append(gs)
     lb, mlb = layernorm_bwd.emit()
     units.append(lb)
@@ -119,6 +120,8 @@ def generate():
     h += [
           "hipError_t lego_grouped_gemm_f16_launch(const void* const*, const void* const*, void* const*, "
           "const int*, int, hipStream_t);",
+          f"hipError_t lego_grouped_gemm_f16_t{GEMM_SMALL_TILE}x{GEMM_SMALL_TILE}_launch(const void* const*, "
+          "const void* const*, void* const*, const int*, int, hipStream_t);",
           f"#define LEGO_GEMM_BM {mg['BM']}", f"#define LEGO_GEMM_BN {mg['BN']}", f"#define LEGO_GEMM_BK {mg['BK']}",
           f"#define LEGO_GEMM_BK_8BIT {GEMM_BK['e5m2']}",
           f"#define LEGO_GROUPED_MAX_GROUPS {mg['MAX_GROUPS']}", ""]

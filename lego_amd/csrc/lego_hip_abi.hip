@@ -241,6 +241,49 @@ int lego_hip_nw_i32(const int* reference, int* matrix, int n, int penalty, void*
   return ok_or(lego_nw_i32_launch(reference, matrix, n, penalty, as_stream(stream)));
 }
 
+namespace {
+// Time of a launch of the grouped kernel, in k-tiles of one workgroup: list scheduling of its
+// tiles, in launch order, on `slots` workgroups that run at once (a tile goes to the slot that
+// frees up first).  tiles[g] tiles of depth[g] k-tiles each.  The slot loads are kept as a
+// sorted list of (load, how many slots) levels, so a group of equal tiles costs a few steps.
+static double grouped_makespan(const long* tiles, const long* depth, int groups, long slots)
+{
+  struct Level { double load; long count; };
+  Level lv[4 * LEGO_GROUPED_MAX_GROUPS + 4];
+  int n = 1;
+  lv[0] = {0.0, slots};
+  for (int g = 0; g < groups; ++g) {
+    long left = tiles[g];
+    const double d = static_cast<double>(depth[g]);
+    while (left > 0) {
+      // the least loaded level takes tiles, one per slot; its slots move up by d
+      const long take = left < lv[0].count ? left : lv[0].count;
+      const double moved = lv[0].load + d;
+      lv[0].count -= take;
+      left -= take;
+      if (lv[0].count == 0) {
+        for (int i = 1; i < n; ++i) lv[i - 1] = lv[i];
+        --n;
+      }
+      // insert (moved, take) keeping the list sorted; merge equal loads
+      int pos = 0;
+      while (pos < n && lv[pos].load < moved) ++pos;
+      if (pos < n && lv[pos].load == moved) {
+        lv[pos].count += take;
+      } else if (n < static_cast<int>(sizeof(lv) / sizeof(lv[0]))) {
+        for (int i = n; i > pos; --i) lv[i] = lv[i - 1];
+        lv[pos] = {moved, take};
+        ++n;
+      } else {
+        lv[n - 1].count += take;        // out of levels (never with <= 64 groups): fold into the top one
+        if (lv[n - 1].load < moved) lv[n - 1].load = moved;
+      }
+    }
+  }
+  return lv[n - 1].load;
+}
+}  // namespace
+
 int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* const* c,
                               const int* sizes3, int groups, void* stream)
 {
@@ -251,7 +294,43 @@ int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* 
     if (!usable(a[g]) || !usable(b[g]) || !usable(c[g])) return kInvalid;
     if (m <= 0 || n <= 0 || k <= 0 || m % 8 || n % 8 || k % LEGO_GEMM_BK) return kInvalid;
   }
-  return ok_or(lego_grouped_gemm_f16_launch(a, b, c, sizes3, groups, as_stream(stream)));
+  // One launch, on 256 x 256 tiles (one workgroup per CU) or on 128 x 128 tiles (four times as many
+  // workgroups of a quarter of the work, two per CU), whichever the estimate below finishes first:
+  // small tiles win when the big ones leave most CUs idle or the last round mostly empty.  Problems
+  // are launched in order of decreasing depth, so the longest tiles start first.  (Splitting the
+  // problems over both kernels was measured and never beat the better of the two single launches.)
+  int order[LEGO_GROUPED_MAX_GROUPS];
+  for (int g = 0; g < groups; ++g) order[g] = g;
+  for (int i = 1; i < groups; ++i) {
+    const int o = order[i];
+    int j = i;
+    while (j > 0 && sizes3[3 * order[j - 1] + 2] < sizes3[3 * o + 2]) { order[j] = order[j - 1]; --j; }
+    order[j] = o;
+  }
+  long big[LEGO_GROUPED_MAX_GROUPS], small[LEGO_GROUPED_MAX_GROUPS], depth[LEGO_GROUPED_MAX_GROUPS];
+  const void* pa[LEGO_GROUPED_MAX_GROUPS];
+  const void* pb[LEGO_GROUPED_MAX_GROUPS];
+  void* pc[LEGO_GROUPED_MAX_GROUPS];
+  int sz[3 * LEGO_GROUPED_MAX_GROUPS];
+  for (int s = 0; s < groups; ++s) {
+    const int g = order[s];
+    const int m = sizes3[3 * g], n = sizes3[3 * g + 1];
+    big[s] = static_cast<long>((m + 255) / 256) * ((n + 255) / 256);
+    small[s] = static_cast<long>((m + 127) / 128) * ((n + 127) / 128);
+    depth[s] = sizes3[3 * g + 2] / LEGO_GEMM_BK;
+    pa[s] = a[g];
+    pb[s] = b[g];
+    pc[s] = c[g];
+    for (int e = 0; e < 3; ++e) sz[3 * s + e] = sizes3[3 * g + e];
+  }
+  const long cus = 256;                 // MI355X
+  // a 128 x 128 tile sharing its CU with another one, against a 256 x 256 tile of the same depth
+  // that has the CU to itself (measured: 45 us against 68 us for 40 k-tiles)
+  const double small_cost = 0.66;
+  const bool use_small = small_cost * grouped_makespan(small, depth, groups, 2 * cus) <
+                         grouped_makespan(big, depth, groups, cus);
+  return ok_or((use_small ? lego_grouped_gemm_f16_t128x128_launch : lego_grouped_gemm_f16_launch)(
+      pa, pb, pc, sz, groups, as_stream(stream)));
 }
 
 int lego_hip_copy16(const void* in, void* out, unsigned long long bytes, void* stream)

@@ -288,5 +288,5 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
     )
     text = template("gemm.hip.j2").render(**params)
     meta = dict(BM=bm, BN=bn, BK=bk, MAX_GROUPS=MAX_GROUPS)
-    launchers = [f"lego_gemm_{dtype}_{variant}{tag}_launch"] + (["lego_grouped_gemm_f16_launch"] if with_grouped else [])
+    launchers = [f"lego_gemm_{dtype}_{variant}{tag}_launch"] + ([f"lego_grouped_gemm_f16{tag}_launch"] if with_grouped else [])
     return Emitted(f"gemm_{dtype}_{variant}{tag}.hip", text, launchers), meta

@@ -386,6 +386,23 @@ def test_grouped_gemm_reference_test_shapes(ops):
         assert _rel_err(c.cpu(), w) <= 1e-2
 
 
+def test_grouped_gemm_many_tiles_unsorted_depths(ops):
+    """The headline grouped problem set at a sixteenth of its depth, in shuffled order: enough
+    256 x 256 tiles for the one-workgroup-per-CU kernel, and the entry point's reordering by depth
+    must hand every result back to its own problem."""
+    print("grouped gemm many tiles, depths unsorted", flush=True)
+    g = _gen(21)
+    shapes = [(1024, 1024, 64), (4096, 1024, 128), (2048, 4096, 64), (4096, 4096, 64), (1024, 4096, 128),
+              (2048, 2048, 64), (1024, 1024, 64), (4096, 2048, 64)]
+    A = [(torch.randn(m, k, generator=g) / math.sqrt(k)).half() for m, n, k in shapes]
+    B = [(torch.randn(k, n, generator=g) / math.sqrt(k)).half() for m, n, k in shapes]
+    want = ok.grouped_gemm(A, B)
+    got = ops.lego_group_gemm_fn([a.cuda() for a in A], [b.cuda() for b in B])
+    for c, w in zip(got, want):
+        assert c.shape == w.shape
+        assert _rel_err(c.cpu(), w) <= 1e-2
+
+
 def test_gemm_rejects_bad_shapes(ops):
     from lego_amd.runtime import LegoHipError
     with pytest.raises(LegoHipError):
