@@ -34,14 +34,16 @@ int lego_hip_transpose_f16(const void* in, void* out, int rows, int cols, void* 
 /* y = softmax(x) over the last dimension of an M x N matrix (fp16 or fp32 in/out), fp32
  * arithmetic.  Replaces softmax(x) (reference: triton_generated/softmax/softmax.py:97-160; the
  * reference's own test is a ragged fp32 1823 x 781 matrix, softmax.py:237-241).
- * Any N up to 16384; rows whose length is a multiple of 16 bytes take the 16-byte-access path. */
+ * Any N up to 32768; rows whose length is a multiple of 16 bytes take the 16-byte-access path,
+ * rows above 16384 elements a whole workgroup of 1024 lanes each. */
 int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream);
 int lego_hip_softmax_f32(const void* x, void* y, int M, int N, void* stream);
 
 /* LayerNorm forward over the last dimension of an M x N matrix; x, y, w, b share one element
  * type (fp16 or fp32), w and b have N elements; mean, rstd are fp32 [M] outputs.  Replaces
  * LEGOLayerNorm.forward / lego_layer_norm (reference:
- * triton_generated/layernorm/layernorm.py:279-307).  Any N up to 16384. */
+ * triton_generated/layernorm/layernorm.py:279-307, whose limit is 64 KiB of row, :291-294).
+ * Any N up to 32768. */
 int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void* b,
                                float* mean, float* rstd, int M, int N, float eps, void* stream);
 int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void* b,
@@ -53,7 +55,8 @@ int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void
  * partial buffers become one fp32 workspace the caller provides (the reference's wrapper
  * allocates its buffers with torch as well): ask for its size first, any 16-byte aligned
  * device buffer of at least that many bytes will do; its contents need no initialisation.
- * N must be a multiple of 8 and at most 16384. */
+ * N must be a multiple of 8 and at most 32768 (the reference's fp16 limit); rows above 16384
+ * elements are read twice (dx by rows, then dw/db by columns). */
 int lego_hip_layernorm_bwd_workspace_bytes(int M, int N, unsigned long long* bytes);
 int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, const float* mean,
                                const float* rstd, void* dx, void* dw, void* db, void* workspace,
@@ -122,7 +125,7 @@ int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* 
                               const int* sizes3, int groups, void* stream);
 
 /* Tuning entry points: as above, with the launch shape chosen by the caller
- * (waves_per_row in {1, 2, 4}; N a multiple of 8).  Used by the benchmark to compare variants. */
+ * (waves_per_row in {1, 2, 4, 16}; N a multiple of 8 and at most 8192 * waves_per_row, 16384 for 4).  Used by the benchmark to compare variants. */
 int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per_row, void* stream);
 int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const void* b,
                                    float* mean, float* rstd, int M, int N, float eps,

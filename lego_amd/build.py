@@ -38,9 +38,10 @@ TRANSPOSE = {
 # (element type, vectorised, waves per row): 16-byte accesses need N % (16/size) == 0; the
 # element-per-access kernels ("s") take any N
 ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f32", True, 1), ("f32", True, 4),
-           ("f16", False, 4), ("f32", False, 4)]
+           ("f16", False, 4), ("f32", False, 4),
+           ("f16", True, 16), ("f32", True, 16), ("f16", False, 16), ("f32", False, 16)]
 ROWWISE_DEFAULT_WAVES = 4
-ROWWISE_MAX_N = 16384
+ROWWISE_MAX_N = rowwise.MAX_N
 GEMM = dict(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8)
 GEMM_SMALL_TILE = 128
 GEMM_SMALL_DTYPES = ("f16", "bf16")     # a 128-byte row of 8-bit elements is too short for their [k][n] rotation
@@ -107,9 +108,12 @@ def generate():
               f"hipError_t lego_layernorm_fwd_{tag}_w{w}_launch(const void*, void*, const void*, const void*, "
               "float*, float*, int, int, float, hipStream_t);"]
     h += [f"#define LEGO_ROWWISE_MAX_N {ROWWISE_MAX_N}",
+          f"#define LEGO_ROWWISE_MAX_N_SMALL_TEAMS {rowwise.MAX_N_SMALL_TEAMS}",
           "// waves per row: one wave keeps short rows free of barriers, four waves keep the",
-          "// register footprint of long rows small enough for full occupancy",
-          f"inline int lego_rowwise_default_wpr(int n) {{ return n <= 2048 ? 1 : {ROWWISE_DEFAULT_WAVES}; }}", ""]
+          "// register footprint of long rows small enough for full occupancy, sixteen (a whole",
+          "// workgroup of 1024 lanes) hold the rows that four cannot",
+          f"inline int lego_rowwise_default_wpr(int n) {{ return n <= 2048 ? 1 : n <= {rowwise.MAX_N_SMALL_TEAMS} ? "
+          f"{ROWWISE_DEFAULT_WAVES} : {rowwise.LONG_ROW_WAVES}; }}", ""]
     h += ["unsigned lego_layernorm_bwd_groups(int M, int N);",
           "hipError_t lego_layernorm_bwd_f16_launch(const void*, const void*, const void*, const float*, const float*, "
           "void*, void*, void*, float*, int, int, hipStream_t);",

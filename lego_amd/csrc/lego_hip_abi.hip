@@ -67,6 +67,7 @@ int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per
     case 1: return ok_or(lego_softmax_f16_w1_launch(x, y, M, N, as_stream(stream)));
     case 2: return ok_or(lego_softmax_f16_w2_launch(x, y, M, N, as_stream(stream)));
     case 4: return ok_or(lego_softmax_f16_w4_launch(x, y, M, N, as_stream(stream)));
+    case 16: return ok_or(lego_softmax_f16_w16_launch(x, y, M, N, as_stream(stream)));
     default: return kInvalid;
   }
 }
@@ -74,16 +75,20 @@ int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per
 int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream)
 {
   if (!usable(x) || !usable(y) || M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N) return kInvalid;
-  if (N % 8) return ok_or(lego_softmax_f16s_w4_launch(x, y, M, N, as_stream(stream)));   // ragged rows
+  const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
+  if (N % 8)   // ragged rows
+    return ok_or((long_row ? lego_softmax_f16s_w16_launch : lego_softmax_f16s_w4_launch)(x, y, M, N, as_stream(stream)));
   return lego_hip_softmax_f16_wpr(x, y, M, N, lego_rowwise_default_wpr(N), stream);
 }
 
 int lego_hip_softmax_f32(const void* x, void* y, int M, int N, void* stream)
 {
   if (!usable(x) || !usable(y) || M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N) return kInvalid;
-  if (N % 4) return ok_or(lego_softmax_f32s_w4_launch(x, y, M, N, as_stream(stream)));   // ragged rows
+  const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
+  if (N % 4)   // ragged rows
+    return ok_or((long_row ? lego_softmax_f32s_w16_launch : lego_softmax_f32s_w4_launch)(x, y, M, N, as_stream(stream)));
   if (N <= 1024) return ok_or(lego_softmax_f32_w1_launch(x, y, M, N, as_stream(stream)));
-  return ok_or(lego_softmax_f32_w4_launch(x, y, M, N, as_stream(stream)));
+  return ok_or((long_row ? lego_softmax_f32_w16_launch : lego_softmax_f32_w4_launch)(x, y, M, N, as_stream(stream)));
 }
 
 int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const void* b,
@@ -96,6 +101,7 @@ int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const 
     case 1: return ok_or(lego_layernorm_fwd_f16_w1_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
     case 2: return ok_or(lego_layernorm_fwd_f16_w2_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
     case 4: return ok_or(lego_layernorm_fwd_f16_w4_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+    case 16: return ok_or(lego_layernorm_fwd_f16_w16_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
     default: return kInvalid;
   }
 }
@@ -105,7 +111,10 @@ int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void
 {
   if (!usable(x) || !usable(y) || !usable(w) || !usable(b) || mean == nullptr || rstd == nullptr) return kInvalid;
   if (M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
-  if (N % 8) return ok_or(lego_layernorm_fwd_f16s_w4_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+  const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
+  if (N % 8)   // ragged rows
+    return ok_or((long_row ? lego_layernorm_fwd_f16s_w16_launch : lego_layernorm_fwd_f16s_w4_launch)(
+        x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
   return lego_hip_layernorm_fwd_f16_wpr(x, y, w, b, mean, rstd, M, N, eps, lego_rowwise_default_wpr(N), stream);
 }
 
@@ -114,9 +123,13 @@ int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void
 {
   if (!usable(x) || !usable(y) || !usable(w) || !usable(b) || mean == nullptr || rstd == nullptr) return kInvalid;
   if (M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
-  if (N % 4) return ok_or(lego_layernorm_fwd_f32s_w4_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+  const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
+  if (N % 4)   // ragged rows
+    return ok_or((long_row ? lego_layernorm_fwd_f32s_w16_launch : lego_layernorm_fwd_f32s_w4_launch)(
+        x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
   if (N <= 1024) return ok_or(lego_layernorm_fwd_f32_w1_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
-  return ok_or(lego_layernorm_fwd_f32_w4_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+  return ok_or((long_row ? lego_layernorm_fwd_f32_w16_launch : lego_layernorm_fwd_f32_w4_launch)(
+      x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
 }
 
 int lego_hip_layernorm_bwd_workspace_bytes(int M, int N, unsigned long long* bytes)

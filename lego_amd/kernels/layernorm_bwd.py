@@ -19,6 +19,11 @@ MAX_GROUPS = 512      # workgroups of stage 1 = rows of the partial buffers
 # (lanes per row, 16-byte vectors per lane): rows of up to 2048, 4096, 8192 and 16384 elements; the
 # longest rows take 512 lanes so that a lane's partial sums still fit its registers
 CONFIGS = ((256, 1), (256, 2), (256, 4), (512, 4))
+# Longer rows (the reference takes fp16 rows of up to 32768 elements, layernorm_triton.py:398-401):
+# 1024 lanes per row leave a lane 128 registers, too few for its partial sums next to the row, so
+# that kernel only writes dx, and dw/db come from a second pass over dy and x by columns.
+LONG = (1024, 4)
+LONG_GROUPS = 64      # row slices of the column pass = rows of its partial buffers
 
 
 def emit():
@@ -29,18 +34,20 @@ def emit():
     X = OrderBy(Row(M, N)).TileBy([M, N / 8], [1, 8])
     P = OrderBy(Row(G, N)).TileBy([G, N / 8], [1, 8])
     params = dict(
-        banner=BANNER, CONFIGS=list(CONFIGS), MAX_GROUPS=MAX_GROUPS,
+        banner=BANNER, CONFIGS=list(CONFIGS), MAX_GROUPS=MAX_GROUPS, LONG=LONG, LONG_GROUPS=LONG_GROUPS,
+        KERNELS=[(th, v, True) for th, v in CONFIGS] + [LONG + (False,)],
+        MAX_N_ACC=max(th * v for th, v in CONFIGS) * 8,
         MAX_N_256=max(v for th, v in CONFIGS if th == 256) * 256 * 8,
         row_layout="OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])[step, wg]",
         x_layout="OrderBy(Row(M, N)).TileBy([M, N/8], [1, 8])[row, v, 0, :]",
         part_layout="OrderBy(Row(G, N)).TileBy([G, N/8], [1, 8])[wg, v, 0, :]",
         row=code(row_e),
         row_base=code(tidy(X[row, 0, 0, 0], {row: (0, M)})).replace("row", "static_cast<size_t>(row)"),
-        vecs={th: code(it * th + t) for th in sorted({th for th, _ in CONFIGS})},
+        vecs={th: code(it * th + t) for th in sorted({th for th, _ in CONFIGS + (LONG,)})},
         vec_off=code(tidy(X[0, v, 0, 0], {v: (0, N / 8)})),
         stat_off=code(OrderBy(Row(M)).TileBy([M])[row,]),
         part_off=code(tidy(P[wg, v, 0, 0], {wg: (0, G), v: (0, N / 8)})).replace("wg", "static_cast<size_t>(wg)"),
     )
     text = template("layernorm_bwd.hip.j2").render(**params)
     return Emitted("layernorm_bwd_f16.hip", text, ["lego_layernorm_bwd_f16_launch"]), dict(
-        MAX_N=max(th * v for th, v in CONFIGS) * 8, MAX_GROUPS=MAX_GROUPS)
+        MAX_N=LONG[0] * LONG[1] * 8, MAX_GROUPS=MAX_GROUPS)

@@ -19,8 +19,10 @@ from __future__ import annotations
 from ..lego import OrderBy, Row
 from .common import BANNER, Emitted, code, idx, size, template, tidy
 
-THREADS = 256
-MAX_N = 16384
+THREADS = 256                  # lanes per workgroup; a team of 16 waves is a workgroup of 1024
+MAX_N = 32768                  # the reference's fp16 LayerNorm limit (64 KiB of row, layernorm_triton.py:335-338)
+MAX_N_SMALL_TEAMS = 16384      # teams of up to four waves; longer rows take sixteen
+LONG_ROW_WAVES = 16
 VPTS = (1, 2, 4, 8, 16, 32, 64)
 
 
@@ -33,7 +35,11 @@ def emit(waves_per_row=1, dtype="f16", vectorised=True):
     EPV = 16 // esize if vectorised else 1
     tag = dtype if vectorised else dtype + "s"
     TEAM = 64 * WPR
-    RPW = THREADS // TEAM                       # rows per workgroup
+    threads = max(THREADS, TEAM)
+    RPW = threads // TEAM                       # rows per workgroup
+    # register footprints: a lane keeps V*EPV fp32 values, at most 128; the sixteen-wave team only
+    # gets the footprints that the smaller teams do not cover
+    lo, hi = (MAX_N_SMALL_TEAMS, MAX_N) if WPR >= LONG_ROW_WAVES else (0, MAX_N_SMALL_TEAMS)
     M, N, NWG = size("M"), size("N"), size("NWG")
     wg, t, it, lane, team, row, v = (idx(n) for n in ("wg", "t", "it", "lane", "team", "row", "v"))
 
@@ -50,9 +56,8 @@ def emit(waves_per_row=1, dtype="f16", vectorised=True):
     stat = OrderBy(Row(M)).TileBy([M])[row,]
 
     params = dict(
-        banner=BANNER, WPR=WPR, TEAM=TEAM, RPW=RPW, THREADS=THREADS,
-        # a lane keeps V*EPV fp32 values: at most 128, and no more footprints than MAX_N needs
-        VPTS=[vp for vp in VPTS if vp * EPV <= 128 and vp * TEAM * EPV <= MAX_N],
+        banner=BANNER, WPR=WPR, TEAM=TEAM, RPW=RPW, THREADS=threads,
+        VPTS=[vp for vp in VPTS if vp * EPV <= 128 and lo < vp * TEAM * EPV <= hi],
         dtype=dtype, elt=elt, EPV=EPV, tag=tag,
         row_layout=f"OrderBy(Row(NWG, {RPW})).TileBy([NWG], [{RPW}])[wg, team]",
         lane_layout=f"OrderBy(Row({RPW}, {TEAM})).TileBy([{RPW}, {TEAM}]).inv(t); vector = it*{TEAM} + lane",

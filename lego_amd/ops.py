@@ -105,7 +105,7 @@ def layer_norm_fwd(x, weight, bias, eps=1e-5, waves_per_row: int | None = None):
 
 
 def layer_norm_bwd(dy, x, weight, mean, rstd):
-    """LayerNorm backward; returns ``(dx, dw, db)``.  fp16, rows of up to 16384 elements."""
+    """LayerNorm backward; returns ``(dx, dw, db)``.  fp16, rows of up to 32768 elements."""
     x_arg = x.reshape(-1, x.shape[-1])
     dy_arg = dy.reshape(-1, dy.shape[-1])
     _check(x_arg, torch.float16, "x")

@@ -136,7 +136,8 @@ def test_softmax_reference_test_shape_fp32(ops):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
-@pytest.mark.parametrize("M,N", [(5, 1), (9, 3), (17, 781), (4, 1000), (3, 4099), (2, 16383), (6, 2048), (3, 16384)])
+@pytest.mark.parametrize("M,N", [(5, 1), (9, 3), (17, 781), (4, 1000), (3, 4099), (2, 16383), (6, 2048), (3, 16384),
+                                 (3, 16392), (2, 20001), (5, 32767), (4, 32768)])
 def test_softmax_ragged_and_fp32(ops, dtype, M, N):
     print(f"softmax {dtype} {M}x{N}", flush=True)
     x = (2.0 * torch.randn(M, N, generator=_gen(2))).to(dtype)
@@ -146,9 +147,15 @@ def test_softmax_ragged_and_fp32(ops, dtype, M, N):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
-@pytest.mark.parametrize("M,N", [(5, 1), (9, 3), (17, 781), (3, 4099), (6, 2048), (3, 16384)])
+@pytest.mark.parametrize("M,N", [(5, 1), (9, 3), (17, 781), (3, 4099), (6, 2048), (3, 16384), (3, 16392), (2, 20001),
+                                 (4, 32768)])
 def test_layernorm_ragged_and_fp32(ops, dtype, M, N):
     print(f"layernorm {dtype} {M}x{N}", flush=True)
+    if N * torch.empty((), dtype=dtype).element_size() > 65536:
+        with pytest.raises(RuntimeError, match="64KB"):    # the reference's limit and message (layernorm.py:293-294)
+            ops.layer_norm_fwd(torch.zeros(M, N, dtype=dtype, device="cuda"), torch.zeros(N, dtype=dtype, device="cuda"),
+                               torch.zeros(N, dtype=dtype, device="cuda"), 1e-5)
+        return
     g = _gen(3)
     x = (2.0 * torch.randn(M, N, generator=g)).to(dtype)
     w = (1 + 0.1 * torch.randn(N, generator=g)).to(dtype)
@@ -160,6 +167,30 @@ def test_layernorm_ragged_and_fp32(ops, dtype, M, N):
     assert torch.allclose(mean.cpu(), want_mean, atol=1e-4, rtol=1e-4)
     if N > 1:
         assert torch.allclose(rstd.cpu(), want_rstd, atol=1e-4, rtol=1e-3)
+
+
+@pytest.mark.parametrize("N", [16392, 30001, 32768])
+def test_layernorm_fp32_long_rows_through_the_c_abi(ops, N):
+    """fp32 rows above 64 KiB: the Python wrapper keeps the reference's limit, the library takes them."""
+    import ctypes
+    from lego_amd import runtime
+    print(f"layernorm fp32 long row {N}", flush=True)
+    M = 5
+    g = _gen(23)
+    x = 2.0 * torch.randn(M, N, generator=g)
+    w = 1 + 0.1 * torch.randn(N, generator=g)
+    b = 0.1 * torch.randn(N, generator=g)
+    want_y, want_mean, want_rstd = ok.layernorm_fwd(x, w, b, 1e-5)
+    xd, wd, bd = x.cuda(), w.cuda(), b.cuda()
+    y = torch.empty_like(xd)
+    mean = torch.empty(M, device="cuda")
+    rstd = torch.empty(M, device="cuda")
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    runtime.call("lego_hip_layernorm_fwd_f32", p(xd), p(y), p(wd), p(bd), p(mean), p(rstd), M, N, 1e-5, None)
+    torch.cuda.synchronize()
+    assert (y.cpu() - want_y).abs().max().item() <= 2e-5
+    assert torch.allclose(mean.cpu(), want_mean, atol=1e-4, rtol=1e-4)
+    assert torch.allclose(rstd.cpu(), want_rstd, atol=1e-4, rtol=1e-3)
 
 
 @pytest.mark.parametrize("wpr", [None, 1, 2, 4])
@@ -224,7 +255,7 @@ def test_layernorm_backward_reference_test(ops):
 
 
 @pytest.mark.parametrize("M,N", [(1, 8), (3, 520), (700, 1024), (513, 2048), (64, 8192), (300, 8200), (129, 15872),
-                                 (40, 16384)])
+                                 (40, 16384), (5, 16392), (300, 24576), (70, 32768)])
 def test_layernorm_backward_matches_oracle(ops, M, N):
     print(f"layernorm backward {M}x{N}", flush=True)
     g = _gen(6)
