@@ -324,6 +324,17 @@ def main():
         kernels["next_lud_f32_4096"] = dict(ms=ms, tflops=(2 / 3) * nl ** 3 / ms / 1e9,
                                             note="time of a matrix copy subtracted; fp32 on the vector ALUs")
         del a0, wk
+        # the size the reference publishes (653.5 ms for its LEGO kernel on an A100,
+        # benchmarks/cuda/lud/PerformanceSummary.txt:24-36)
+        nl = 16384
+        a0 = torch.rand(nl, nl, generator=gen(11)).to(dev)
+        a0.diagonal().add_(float(nl))
+        wk = torch.empty_like(a0)
+        ms = timed(luf, steps=2, warmup=1) - timed(lambda: wk.copy_(a0), steps=2, warmup=1)
+        kernels["next_lud_f32_16384"] = dict(ms=ms, tflops=(2 / 3) * nl ** 3 / ms / 1e9,
+                                             reference_ms_a100=653.5,
+                                             note="time of a matrix copy subtracted; 256 block steps of three launches")
+        del a0, wk
 
     # ---- CPU baseline: the oracle on a bounded panel of the headline matrix ------------------------------
     cpu = None
