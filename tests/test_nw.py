@@ -35,9 +35,24 @@ def test_oracle_closed_form_without_substitution_scores():
     assert np.array_equal(got, -np.abs(i - j) * 7)
 
 
+def test_rotation_through_lds_is_free_of_bank_conflicts():
+    """Slot k of lane tx is row (k - tx) mod 64 of column tx: in the kernel's LDS tile the 64 lanes
+    of every such access, and of every row access, fall into 64 different banks."""
+    b = nw.B
+    i, j = sp.symbols("i j", integer=True, nonnegative=True)
+    f = sp.lambdify([i, j], nw.rotation_layout()[i, j], "math")
+    words = set()
+    for k in range(b):
+        slots = [int(f((k - tx) % b, tx)) for tx in range(b)]
+        assert len({w % 64 for w in slots}) == 64
+        words.update(slots)
+        assert len({int(f(k, tx)) % 64 for tx in range(b)}) == 64
+    assert words == set(range(b * b))
+
+
 def test_tile_layout_is_the_anti_diagonal_enumeration():
-    """The LDS layout of the kernel: a bijection of the 64 x 64 tile in which the cells of one
-    anti-diagonal are consecutive and ordered by row."""
+    """The reference's layout of the tile (nw_sympy.py:9-11): a bijection of the 64 x 64 tile in
+    which the cells of one anti-diagonal are consecutive and ordered by row."""
     b = nw.B
     i, j = sp.symbols("i j", integer=True, nonnegative=True)
     f = sp.lambdify([i, j], nw.tile_layout()[i, j], "math")
