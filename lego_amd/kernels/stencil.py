@@ -17,10 +17,11 @@ that every index is in range, prints ``... + 64*i + 64*i_diff + ...`` for the br
 brick.  Here a neighbour is addressed by its global coordinates, ``L[x/B, y/B, z/B, x%B, y%B, z%B]``,
 so both storage orders give the stencil's result.
 
-A workgroup of 512 lanes is one brick; lane ``t`` is point ``Row(B, B, B).inv(t)`` of it, last
-coordinate fastest, so a wavefront touches 64 consecutive floats of a brick (bricks storage) or
-eight 32-byte runs (row-major storage).  The brick and a shell of ``radius`` points around it
-are staged in LDS once; the neighbours of a point are read from there.
+A wavefront is one brick; lane ``l`` owns row ``Row(B, B).inv(l)`` of it, the ``B`` points along the
+last axis: 32 contiguous bytes in both storage orders, kept in registers.  A wavefront's access
+to one row of every lane is the whole 2 KiB brick (bricks storage) or 64 runs of 32 bytes
+(row-major storage).  The neighbours along the last axis are the lane's own registers plus
+``radius`` points on either side; the other neighbours are whole rows again, fetched the same way.
 """
 from __future__ import annotations
 
@@ -29,6 +30,10 @@ from .common import BANNER, Emitted, code, idx, size, template, tidy
 
 B = 8
 MAX_RADIUS = 3        # the coefficient cube is 8 x 8 x 8: offsets -3..3 plus one unused plane
+WAVES = 4             # bricks per workgroup
+# words per row of the shell in LDS: 16 hold a row (3 + 8 + 3 points, 16-byte aligned), 20 spread the
+# 16-byte reads of eight neighbouring lanes over different banks
+ROW_WORDS = 20
 
 
 def layouts(nb):
@@ -44,23 +49,26 @@ def emit():
     x, y, z = idx("x"), idx("y"), idx("z")
     a, b_, c_ = idx("ca"), idx("cb"), idx("cc")
     bxyz = OrderBy(Row(nb, nb, nb)).TileBy([nb, nb, nb]).inv(wg)
-    ijk = OrderBy(Row(B, B, B)).TileBy([B, B, B]).inv(t)
+    ij = OrderBy(Row(B, B)).TileBy([B, B]).inv(t)
     rng = {x: (0, B * nb), y: (0, B * nb), z: (0, B * nb)}
     at = [code(tidy(L[x // B, y // B, z // B, x % B, y % B, z % B], rng)) for L in layouts(nb)]
     coeff = OrderBy(Row(8, 8, 8)).TileBy([8, 8, 8])[a, b_, c_]
-    # the shell cube in LDS: row-major H x H x H, H a compile-time constant of the kernel
-    H, h, hx, hy, hz = size("H"), idx("h"), idx("hx"), idx("hy"), idx("hz")
-    shell = OrderBy(Row(H, H, H)).TileBy([H, H, H])
-    halo_inv = [code(tidy(e, {h: (0, H * H * H)})) for e in shell.inv(h)]
-    halo_at = code(tidy(shell[hx, hy, hz], {hx: (0, H), hy: (0, H), hz: (0, H)}))
+    # the rows of a brick and its shell in LDS: H x H rows of ROW_WORDS words, H a compile-time constant
+    H, h, hx, hy = size("H"), idx("h"), idx("hx"), idx("hy")
+    shell_rows = OrderBy(Row(H, H)).TileBy([H, H])
+    shell_inv = [code(tidy(e, {h: (0, H * H)})) for e in shell_rows.inv(h)]
+    shell = OrderBy(Row(H, H, ROW_WORDS)).TileBy([H, H, ROW_WORDS])
+    shell_row = code(tidy(shell[hx, hy, 0], {hx: (0, H), hy: (0, H)}))
     params = dict(
-        banner=BANNER, B=B, MAX_RADIUS=MAX_RADIUS,
+        shell_layout=f"OrderBy(Row(H, H, {ROW_WORDS})).TileBy([H, H, {ROW_WORDS}])[hx, hy, word]",
+        shell_inv=shell_inv, shell_row=shell_row, ROW_WORDS=ROW_WORDS,
+        banner=BANNER, B=B, MAX_RADIUS=MAX_RADIUS, WAVES=WAVES,
+        row_layout=f"Row({B}, {B})",
         normal_layout=f"OrderBy(Row(N, N, N)).TileBy([N/{B}]*3, [{B}]*3)[x/{B}, y/{B}, z/{B}, x%{B}, y%{B}, z%{B}]",
         bricks_layout=f"OrderBy(Row(N/{B}, N/{B}, N/{B}), Row({B}, {B}, {B})).TileBy([N/{B}]*3, [{B}]*3)[x/{B}, ...]",
         brick=[code(tidy(e, {wg: (0, nb * nb * nb)})) for e in bxyz],
-        point=[code(tidy(e, {t: (0, B * B * B)})) for e in ijk],
+        row=[code(tidy(e, {t: (0, B * B)})) for e in ij],
         at_normal=at[0], at_bricks=at[1], coeff=code(coeff),
-        halo_layout="OrderBy(Row(H, H, H)).TileBy([H, H, H])", halo_inv=halo_inv, halo_at=halo_at,
     )
     text = template("stencil.hip.j2").render(**params)
     return Emitted("stencil_f32.hip", text, ["lego_stencil_f32_launch"]), dict(B=B, MAX_RADIUS=MAX_RADIUS)
