@@ -322,7 +322,7 @@ def main():
             runtime.call("lego_hip_lud_f32", p(wk), nl, stream)
         ms = timed(luf, steps=3, warmup=1) - timed(lambda: wk.copy_(a0), steps=3, warmup=1)
         kernels["next_lud_f32_4096"] = dict(ms=ms, tflops=(2 / 3) * nl ** 3 / ms / 1e9,
-                                            note="time of a matrix copy subtracted; fp32 on the vector ALUs")
+                                            note="time of a matrix copy subtracted")
         del a0, wk
         # the size the reference publishes (653.5 ms for its LEGO kernel on an A100,
         # benchmarks/cuda/lud/PerformanceSummary.txt:24-36)
