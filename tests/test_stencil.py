@@ -82,7 +82,7 @@ def _from_bricks(y, order):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("bricks", [False, True])
-@pytest.mark.parametrize("n,radius", [(16, 1), (64, 1), (64, 2), (32, 3), (128, 1)])
+@pytest.mark.parametrize("n,radius", [(8, 1), (8, 3), (16, 1), (24, 2), (64, 1), (64, 2), (32, 3), (128, 1)])
 def test_gpu_f3d_matches_oracle(n, radius, bricks):
     from lego_amd import ops
     print(f"f3d n={n} radius={radius} bricks={bricks}", flush=True)
@@ -99,7 +99,7 @@ def test_gpu_f3d_matches_oracle(n, radius, bricks):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("bricks", [False, True])
-@pytest.mark.parametrize("n,radius", [(16, 1), (64, 2), (64, 3), (128, 1)])
+@pytest.mark.parametrize("n,radius", [(8, 1), (8, 3), (16, 1), (24, 3), (64, 2), (64, 3), (128, 1)])
 def test_gpu_laplacian_matches_oracle(n, radius, bricks):
     from lego_amd import ops
     print(f"laplacian n={n} radius={radius} bricks={bricks}", flush=True)
