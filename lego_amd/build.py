@@ -64,6 +64,7 @@ def generate():
             tmeta.setdefault(dtype, []).append(meta)
     units.append(transpose.emit_any())
     units += [rowwise.emit(w, dtype, vec) for dtype, vec, w in ROWWISE]
+    units.append(rowwise.emit_long())
     for dtype in GEMM_DTYPES:
         for ta in (False, True):
             for tb in (False, True):
@@ -107,7 +108,9 @@ def generate():
         h += [f"hipError_t lego_softmax_{tag}_w{w}_launch(const void*, void*, int, int, hipStream_t);",
               f"hipError_t lego_layernorm_fwd_{tag}_w{w}_launch(const void*, void*, const void*, const void*, "
               "float*, float*, int, int, float, hipStream_t);"]
-    h += [f"#define LEGO_ROWWISE_MAX_N {ROWWISE_MAX_N}",
+    h += ["hipError_t lego_softmax_long_f16_launch(const void*, void*, int, int, hipStream_t);",
+          "hipError_t lego_softmax_long_f32_launch(const void*, void*, int, int, hipStream_t);",
+          f"#define LEGO_ROWWISE_MAX_N {ROWWISE_MAX_N}",
           f"#define LEGO_ROWWISE_MAX_N_SMALL_TEAMS {rowwise.MAX_N_SMALL_TEAMS}",
           "// waves per row: one wave keeps short rows free of barriers, four waves keep the",
           "// register footprint of long rows small enough for full occupancy, sixteen (a whole",

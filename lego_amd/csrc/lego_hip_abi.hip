@@ -74,7 +74,8 @@ int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per
 
 int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream)
 {
-  if (!usable(x) || !usable(y) || M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N) return kInvalid;
+  if (!usable(x) || !usable(y) || M <= 0 || N <= 0) return kInvalid;
+  if (N > LEGO_ROWWISE_MAX_N) return ok_or(lego_softmax_long_f16_launch(x, y, M, N, as_stream(stream)));   // two passes
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 8)   // ragged rows
     return ok_or((long_row ? lego_softmax_f16s_w16_launch : lego_softmax_f16s_w4_launch)(x, y, M, N, as_stream(stream)));
@@ -83,7 +84,8 @@ int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream)
 
 int lego_hip_softmax_f32(const void* x, void* y, int M, int N, void* stream)
 {
-  if (!usable(x) || !usable(y) || M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N) return kInvalid;
+  if (!usable(x) || !usable(y) || M <= 0 || N <= 0) return kInvalid;
+  if (N > LEGO_ROWWISE_MAX_N) return ok_or(lego_softmax_long_f32_launch(x, y, M, N, as_stream(stream)));   // two passes
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 4)   // ragged rows
     return ok_or((long_row ? lego_softmax_f32s_w16_launch : lego_softmax_f32s_w4_launch)(x, y, M, N, as_stream(stream)));

@@ -69,3 +69,22 @@ def emit(waves_per_row=1, dtype="f16", vectorised=True):
     text = template("rowwise.hip.j2").render(**params)
     return Emitted(f"rowwise_{tag}_w{WPR}.hip", text,
                    [f"lego_softmax_{tag}_w{WPR}_launch", f"lego_layernorm_fwd_{tag}_w{WPR}_launch"])
+
+
+def emit_long():
+    """Softmax of rows of any length: one workgroup of 1024 lanes per row, two passes over the row
+    (a running maximum and rescaled sum, then the normalised exponentials)."""
+    M, N = size("M"), size("N")
+    row, v = idx("row"), idx("v")
+    variants, vec_off = [], {}
+    for dtype, (elt, esize) in (("f16", ("_Float16", 2)), ("f32", ("float", 4))):
+        epv = 16 // esize
+        variants.append((dtype, elt, epv))
+        X = OrderBy(Row(M, N)).TileBy([M, N / epv], [1, epv])
+        vec_off[epv] = code(tidy(X[0, v, 0, 0], {v: (0, N / epv)}))
+        row_base = tidy(X[row, 0, 0, 0], {row: (0, M)})
+    text = template("softmax_long.hip.j2").render(
+        banner=BANNER, THREADS=1024, VARIANTS=variants, vec_off=vec_off,
+        row_base=code(row_base).replace("row", "static_cast<size_t>(row)"),
+        x_layout="OrderBy(Row(M, N)).TileBy([M, N/EPV], [1, EPV])[row, v, 0, :]")
+    return Emitted("softmax_long.hip", text, ["lego_softmax_long_f16_launch", "lego_softmax_long_f32_launch"])

@@ -124,6 +124,21 @@ def test_softmax_matches_oracle(ops, M, N, wpr):
     assert torch.allclose(got.float().sum(-1), torch.ones(M), atol=2e-2)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("M,N", [(3, 32776), (2, 50257), (5, 65536), (2, 131072), (1, 200003)])
+def test_softmax_rows_read_twice(ops, dtype, M, N):
+    """Rows above 32768 elements (vocabulary-sized rows among them): running maximum and sum, then
+    a second pass."""
+    print(f"softmax long rows {dtype} {M}x{N}", flush=True)
+    x = (2.0 * torch.randn(M, N, generator=_gen(24))).to(dtype)
+    x[0, 7] = 11.0               # a maximum that arrives early ...
+    x[-1, N - 3] = 12.5          # ... and one that arrives late
+    want = ok.softmax(x)
+    got = ops.softmax(x.cuda()).cpu()
+    assert (got.float() - want.float()).abs().max().item() <= (TOL if dtype == torch.float16 else 1e-6)
+    assert torch.allclose(got.float().sum(-1), torch.ones(M), atol=2e-2 if dtype == torch.float16 else 1e-4)
+
+
 def test_softmax_reference_test_shape_fp32(ops):
     """The reference's own check (softmax.py:237-241): seed 0, x = randn(1823, 781) in fp32,
     compared with torch.softmax at allclose's default tolerance."""
