@@ -34,7 +34,7 @@ int lego_hip_transpose_f16(const void* in, void* out, int rows, int cols, void* 
 /* y = softmax(x) over the last dimension of an M x N matrix (fp16 or fp32 in/out), fp32
  * arithmetic.  Replaces softmax(x) (reference: triton_generated/softmax/softmax.py:97-160; the
  * reference's own test is a ragged fp32 1823 x 781 matrix, softmax.py:237-241).
- * Any N; rows whose length is a multiple of 16 bytes take the 16-byte-access path, rows above
+ * Any N; rows that are not whole 16-byte vectors are split at their 16-byte boundaries, rows above
  * 16384 elements a whole workgroup of 1024 lanes each, rows above 32768 elements are read twice
  * (the reference keeps a whole row in one block whatever its length, softmax.py:104). */
 int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream);

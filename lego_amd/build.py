@@ -38,7 +38,7 @@ TRANSPOSE = {
 # (element type, vectorised, waves per row): 16-byte accesses need N % (16/size) == 0; the
 # element-per-access kernels ("s") take any N
 ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f32", True, 1), ("f32", True, 4),
-           ("f16", False, 4), ("f32", False, 4),
+           ("f16", False, 1), ("f32", False, 1), ("f16", False, 4), ("f32", False, 4),
            ("f16", True, 16), ("f32", True, 16), ("f16", False, 16), ("f32", False, 16)]
 ROWWISE_DEFAULT_WAVES = 4
 ROWWISE_MAX_N = rowwise.MAX_N

@@ -78,7 +78,9 @@ int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream)
   if (N > LEGO_ROWWISE_MAX_N) return ok_or(lego_softmax_long_f16_launch(x, y, M, N, as_stream(stream)));   // two passes
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 8)   // ragged rows
-    return ok_or((long_row ? lego_softmax_f16s_w16_launch : lego_softmax_f16s_w4_launch)(x, y, M, N, as_stream(stream)));
+    return ok_or((long_row ? lego_softmax_f16s_w16_launch : lego_rowwise_default_wpr(N) == 1 ? lego_softmax_f16s_w1_launch
+                                                                                           : lego_softmax_f16s_w4_launch)(
+        x, y, M, N, as_stream(stream)));
   return lego_hip_softmax_f16_wpr(x, y, M, N, lego_rowwise_default_wpr(N), stream);
 }
 
@@ -88,7 +90,8 @@ int lego_hip_softmax_f32(const void* x, void* y, int M, int N, void* stream)
   if (N > LEGO_ROWWISE_MAX_N) return ok_or(lego_softmax_long_f32_launch(x, y, M, N, as_stream(stream)));   // two passes
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 4)   // ragged rows
-    return ok_or((long_row ? lego_softmax_f32s_w16_launch : lego_softmax_f32s_w4_launch)(x, y, M, N, as_stream(stream)));
+    return ok_or((long_row ? lego_softmax_f32s_w16_launch : N <= 1024 ? lego_softmax_f32s_w1_launch
+                                                                      : lego_softmax_f32s_w4_launch)(x, y, M, N, as_stream(stream)));
   if (N <= 1024) return ok_or(lego_softmax_f32_w1_launch(x, y, M, N, as_stream(stream)));
   return ok_or((long_row ? lego_softmax_f32_w16_launch : lego_softmax_f32_w4_launch)(x, y, M, N, as_stream(stream)));
 }
@@ -115,7 +118,8 @@ int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void
   if (M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 8)   // ragged rows
-    return ok_or((long_row ? lego_layernorm_fwd_f16s_w16_launch : lego_layernorm_fwd_f16s_w4_launch)(
+    return ok_or((long_row ? lego_layernorm_fwd_f16s_w16_launch : lego_rowwise_default_wpr(N) == 1 ? lego_layernorm_fwd_f16s_w1_launch
+                                                                                                 : lego_layernorm_fwd_f16s_w4_launch)(
         x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
   return lego_hip_layernorm_fwd_f16_wpr(x, y, w, b, mean, rstd, M, N, eps, lego_rowwise_default_wpr(N), stream);
 }
@@ -127,7 +131,8 @@ int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void
   if (M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 4)   // ragged rows
-    return ok_or((long_row ? lego_layernorm_fwd_f32s_w16_launch : lego_layernorm_fwd_f32s_w4_launch)(
+    return ok_or((long_row ? lego_layernorm_fwd_f32s_w16_launch : N <= 1024 ? lego_layernorm_fwd_f32s_w1_launch
+                                                                            : lego_layernorm_fwd_f32s_w4_launch)(
         x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
   if (N <= 1024) return ok_or(lego_layernorm_fwd_f32_w1_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
   return ok_or((long_row ? lego_layernorm_fwd_f32_w16_launch : lego_layernorm_fwd_f32_w4_launch)(

@@ -28,11 +28,12 @@ VPTS = (1, 2, 4, 8, 16, 32, 64)
 
 def emit(waves_per_row=1, dtype="f16", vectorised=True):
     """One translation unit: every register footprint ``V`` of one (waves per row, element type,
-    access width) combination.  ``vectorised=False`` emits the element-per-access kernels that
-    take rows of any length and alignment (the reference's own softmax test is 1823 x 781)."""
+    access width) combination.  ``vectorised=False`` emits the kernels that take rows of any length
+    and alignment (the reference's own softmax test is 1823 x 781): the elements before a row's
+    first 16-byte boundary and after its last whole vector go one per lane, the rest as vectors."""
     WPR = waves_per_row
     elt, esize = {"f16": ("_Float16", 2), "f32": ("float", 4)}[dtype]
-    EPV = 16 // esize if vectorised else 1
+    EPV = 16 // esize
     tag = dtype if vectorised else dtype + "s"
     TEAM = 64 * WPR
     threads = max(THREADS, TEAM)
@@ -58,7 +59,7 @@ def emit(waves_per_row=1, dtype="f16", vectorised=True):
     params = dict(
         banner=BANNER, WPR=WPR, TEAM=TEAM, RPW=RPW, THREADS=threads,
         VPTS=[vp for vp in VPTS if vp * EPV <= 128 and lo < vp * TEAM * EPV <= hi],
-        dtype=dtype, elt=elt, EPV=EPV, tag=tag,
+        dtype=dtype, elt=elt, EPV=EPV, ESIZE=esize, RAGGED=not vectorised, tag=tag,
         row_layout=f"OrderBy(Row(NWG, {RPW})).TileBy([NWG], [{RPW}])[wg, team]",
         lane_layout=f"OrderBy(Row({RPW}, {TEAM})).TileBy([{RPW}, {TEAM}]).inv(t); vector = it*{TEAM} + lane",
         x_layout=f"OrderBy(Row(M, N)).TileBy([M, N/{EPV}], [1, {EPV}])[row, v, 0, :]",
