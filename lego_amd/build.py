@@ -25,15 +25,17 @@ OBJ_DIR = LIB_DIR / "obj"
 
 # the tilings the library is built with
 # Per element type, in order of preference: the fastest tiling for shapes that its windows
-# divide, a wide macro tile in skewed ("diag") order, and a 64x64 one for shapes the wide tile
-# does not divide.
+# divide, a wide macro tile in skewed ("diag") order, a 64x64 one for shapes the wide tile
+# does not divide, and the wide tile with edge tests for shapes in whole 16-byte vectors.
 TRANSPOSE = {
     "f32": [dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 32, 8), max_bytes=256 << 20),
             dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag"),
-            dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag")],
+            dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag"),
+            dict(dtype="f32", tile=(32, 32), group=(2, 4), order="diag", edge=True)],
     "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 128, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag"),
-            dict(dtype="f16", tile=(64, 64), group=(1, 1), order="diag")],
+            dict(dtype="f16", tile=(64, 64), group=(1, 1), order="diag"),
+            dict(dtype="f16", tile=(64, 64), group=(2, 2), order="diag", edge=True)],
 }
 # (element type, vectorised, waves per row): 16-byte accesses need N % (16/size) == 0; the
 # element-per-access kernels ("s") take any N
@@ -59,6 +61,9 @@ def generate():
             max_bytes = cfg.pop("max_bytes", None)   # only for matrices that fit the last-level cache
             unit, meta = transpose.emit(**cfg, suffix="")
             meta["max_bytes"] = max_bytes
+            if cfg.get("edge"):
+                vec = 4 if dtype == "f32" else 8
+                meta["row_multiple"] = meta["col_multiple"] = vec
             unit.filename = meta["kernel"].replace("lego_", "", 1) + ".hip"
             units.append(unit)
             tmeta.setdefault(dtype, []).append(meta)

@@ -132,8 +132,10 @@ def tile_order(order, n_bi, n_bj, wg):
     raise ValueError(order)
 
 
-def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix=""):
-    """HIP translation unit for one element type and one tiling."""
+def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix="", edge=False):
+    """HIP translation unit for one element type and one tiling.  ``edge``: the shape need not be
+    a whole number of macro tiles, only of 16-byte vectors in both directions; vectors past the
+    edge are skipped."""
     elt, esize = {"f32": ("float", 4), "f16": ("_Float16", 2)}[dtype]
     vec = 16 // esize                       # elements per 16-byte vector
     (TR, TC), (MR, MC) = tile, group
@@ -177,6 +179,9 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix=""):
     v2 = OrderBy(Row(KD, SR // rows_per_read)).TileBy([KD, SR // rows_per_read]).inv(it * THREADS + t)
     v2 = [tidy(x, {t: (0, THREADS), it: (0, P2)}) for x in v2]
 
+    if edge:
+        assert not windowed
+        suffix = f"{suffix}_edge"
     rng1 = {r: (0, SR), cv: (0, SC // vec), e: (0, 4)}
     rng2 = {k: (0, KD), rv: (0, SR // rows_per_read)}
     cols_per_word = 4 // esize
@@ -195,7 +200,16 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix=""):
         lds_load1=code(tidy(lds[k, rv * rows_per_read + 4], rng2)) if esize == 2 else "",
         dst_off0=code(in_tile(dst, rv * rows_per_read, k * cols_per_word, rng2)),
         dst_off1=code(in_tile(dst, rv * rows_per_read, k * cols_per_word + 1, rng2)) if esize == 2 else "",
-        grid=f"static_cast<unsigned>(rows / {SR}) * static_cast<unsigned>(cols / {SC})",
+        grid=(f"static_cast<unsigned>((rows + {SR - 1}) / {SR}) * static_cast<unsigned>((cols + {SC - 1}) / {SC})" if edge
+              else f"static_cast<unsigned>(rows / {SR}) * static_cast<unsigned>(cols / {SC})"),
+        edge=edge,
+        # matrix coordinates of the vectors, for the edge tests: source (row, first column) in phase 1,
+        # destination (row = source column, first column = source row) in phase 2
+        p1_row=code(tidy(OrderBy(Row(nBi, SR)).TileBy([nBi], [SR])[Bi, r], {r: (0, SR)})),
+        p1_col=code(tidy(OrderBy(Row(nBj, SC // vec, vec)).TileBy([nBj], [SC // vec], [vec])[Bj, cv, 0], {cv: (0, SC // vec)})),
+        p2_row0=code(tidy(OrderBy(Row(nBj, KD, cols_per_word)).TileBy([nBj], [KD], [cols_per_word])[Bj, k, 0], {k: (0, KD)})),
+        p2_col=code(tidy(OrderBy(Row(nBi, SR // rows_per_read, rows_per_read)).TileBy([nBi], [SR // rows_per_read], [rows_per_read])[Bi, rv, 0],
+                         {rv: (0, SR // rows_per_read)})),
     )
     text = template("transpose.hip.j2").render(**params)
     return Emitted(f"transpose_{dtype}{suffix}.hip", text, [params["kernel"] + "_launch"]), dict(

@@ -73,9 +73,14 @@ def test_transpose_moves_bits_of_any_2_or_4_byte_type(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype,rows,cols", [(torch.float32, 100, 64), (torch.float32, 32, 64), (torch.float32, 1, 1),
-                                             (torch.float16, 1823, 781), (torch.float16, 65, 4097), (torch.float32, 777, 3)])
+                                             (torch.float16, 1823, 781), (torch.float16, 65, 4097), (torch.float32, 777, 3),
+                                             (torch.float16, 8, 8), (torch.float16, 72, 264), (torch.float16, 1000, 520),
+                                             (torch.float16, 4104, 1096), (torch.float16, 64, 8), (torch.float16, 8, 1024),
+                                             (torch.float32, 4, 4), (torch.float32, 36, 260), (torch.float32, 1004, 516),
+                                             (torch.float32, 2052, 4100)])
 def test_transpose_of_any_shape(ops, dtype, rows, cols):
-    """Shapes no vectorised tiling divides go through the one-element-per-access kernel."""
+    """Shapes no tiling divides: in whole 16-byte vectors both ways they take the wide tile with edge
+    tests, otherwise the one-element-per-access kernel."""
     print(f"transpose (any shape) {dtype} {rows}x{cols}", flush=True)
     x = (torch.rand(rows, cols, generator=_gen(4)) * 2 - 1).to(dtype)
     want = ok.transpose(x, 1, 1)
