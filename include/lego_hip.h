@@ -57,8 +57,8 @@ int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void
  * partial buffers become one fp32 workspace the caller provides (the reference's wrapper
  * allocates its buffers with torch as well): ask for its size first, any 16-byte aligned
  * device buffer of at least that many bytes will do; its contents need no initialisation.
- * N must be a multiple of 8 and at most 32768 (the reference's fp16 limit); rows above 16384
- * elements are read twice (dx by rows, then dw/db by columns). */
+ * Any N up to 32768 (the reference's fp16 limit); rows above 16384 elements and rows whose length
+ * is not a multiple of 8 are read twice (dx by rows, then dw/db by columns). */
 int lego_hip_layernorm_bwd_workspace_bytes(int M, int N, unsigned long long* bytes);
 int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, const float* mean,
                                const float* rstd, void* dx, void* dw, void* db, void* workspace,

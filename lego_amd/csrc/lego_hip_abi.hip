@@ -141,8 +141,9 @@ int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void
 
 int lego_hip_layernorm_bwd_workspace_bytes(int M, int N, unsigned long long* bytes)
 {
-  if (bytes == nullptr || M <= 0 || N <= 0 || N % 8 || N > LEGO_LAYERNORM_BWD_MAX_N) return kInvalid;
-  *bytes = 2ull * lego_layernorm_bwd_groups(M, N) * static_cast<unsigned long long>(N) * sizeof(float);
+  if (bytes == nullptr || M <= 0 || N <= 0 || N > LEGO_LAYERNORM_BWD_MAX_N) return kInvalid;
+  const unsigned long long pitch = (static_cast<unsigned long long>(N) + 7) / 8 * 8;
+  *bytes = 2ull * lego_layernorm_bwd_groups(M, N) * pitch * sizeof(float);
   return 0;
 }
 

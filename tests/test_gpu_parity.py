@@ -275,7 +275,8 @@ def test_layernorm_backward_reference_test(ops):
 
 
 @pytest.mark.parametrize("M,N", [(1, 8), (3, 520), (700, 1024), (513, 2048), (64, 8192), (300, 8200), (129, 15872),
-                                 (40, 16384), (5, 16392), (300, 24576), (70, 32768)])
+                                 (40, 16384), (5, 16392), (300, 24576), (70, 32768),
+                                 (3, 1), (5, 7), (17, 781), (130, 1000), (9, 4099), (4, 20001), (3, 32767)])
 def test_layernorm_backward_matches_oracle(ops, M, N):
     print(f"layernorm backward {M}x{N}", flush=True)
     g = _gen(6)
