@@ -455,6 +455,27 @@ def test_grouped_gemm_many_tiles_unsorted_depths(ops):
         assert _rel_err(c.cpu(), w) <= 1e-2
 
 
+def test_kernels_run_on_the_callers_stream(ops):
+    """The wrappers enqueue on torch's current stream: work issued on a side stream is ordered after that
+    stream's earlier work (the input is produced there) and is complete once the stream is."""
+    print("side stream", flush=True)
+    side = torch.cuda.Stream()          # default priority
+    g = _gen(25)
+    x_host = (2.0 * torch.randn(512, 4096, generator=g)).half()
+    a_host = (torch.randn(512, 256, generator=g) / 16).half()
+    b_host = (torch.randn(256, 512, generator=g) / 16).half()
+    with torch.cuda.stream(side):
+        x = x_host.cuda(non_blocking=True) * 1.0          # produced on the side stream
+        y = ops.softmax(x)
+        t = ops.transpose(y)
+        c = ops.matmul(a_host.cuda(non_blocking=True), b_host.cuda(non_blocking=True))
+    side.synchronize()
+    want = ok.softmax(x_host)
+    assert (y.cpu().float() - want.float()).abs().max().item() <= TOL
+    assert torch.equal(t.cpu(), y.cpu().t().contiguous())
+    assert _rel_err(c.cpu(), ok.gemm(a_host, b_host)) <= 1e-2
+
+
 def test_gemm_rejects_bad_shapes(ops):
     from lego_amd.runtime import LegoHipError
     with pytest.raises(LegoHipError):
