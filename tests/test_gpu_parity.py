@@ -476,6 +476,42 @@ def test_kernels_run_on_the_callers_stream(ops):
     assert _rel_err(c.cpu(), ok.gemm(a_host, b_host)) <= 1e-2
 
 
+def test_entry_points_replay_from_a_hip_graph(ops):
+    """Nothing behind the C ABI allocates, synchronises or keeps state, so a chain of calls can be
+    captured once and replayed: every replay, on new input, matches the eager result."""
+    print("graph capture and replay", flush=True)
+    g = _gen(26)
+    M, N = 256, 2048
+    x = torch.zeros(M, N, dtype=torch.half, device="cuda")
+    w = (1 + 0.1 * torch.randn(N, generator=g)).half().cuda()
+    b = (0.1 * torch.randn(N, generator=g)).half().cuda()
+    wm = (torch.randn(N, 512, generator=g) / math.sqrt(N)).half().cuda()
+
+    def chain(inp):
+        y, _, _ = ops.layer_norm_fwd(inp, w, b, 1e-5)
+        z = ops.matmul(y, wm)
+        return ops.transpose(ops.softmax(z))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        chain(x)                         # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = chain(x)
+    for trial in range(3):
+        fresh = (2.0 * torch.randn(M, N, generator=g)).half().cuda()
+        x.copy_(fresh)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        want = chain(fresh)              # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), trial
+
+
 def test_gemm_rejects_bad_shapes(ops):
     from lego_amd.runtime import LegoHipError
     with pytest.raises(LegoHipError):
