@@ -512,6 +512,26 @@ def test_entry_points_replay_from_a_hip_graph(ops):
         assert torch.equal(got, want), trial
 
 
+def test_gemm_offsets_beyond_32_bits(ops):
+    """Operands and results of more than 2^32 elements: tile offsets are 64-bit.  The last row tile,
+    whose offset in A (first case) or in C (second case) does not fit 32 bits, is checked against the oracle."""
+    print("gemm with more than 2^32 elements per matrix", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(27)
+    M, K, N = 65536 + 256, 65536, 256
+    a = torch.empty(M, K, device="cuda", dtype=torch.half).normal_(0, 1 / 256, generator=g)
+    b = torch.empty(K, N, device="cuda", dtype=torch.half).normal_(0, 1 / 256, generator=g)
+    c = ops.matmul(a, b)
+    for rows in (slice(0, 256), slice(M - 256, M)):
+        assert _rel_err(c[rows].cpu(), ok.gemm(a[rows].cpu(), b.cpu())) <= 1e-2
+    del a, b, c
+    M, K, N = 65536 + 256, 64, 65536
+    a = torch.empty(M, K, device="cuda", dtype=torch.half).normal_(0, 1 / 8, generator=g)
+    b = torch.empty(K, N, device="cuda", dtype=torch.half).normal_(0, 1 / 8, generator=g)
+    c = ops.matmul(a, b)
+    for rows in (slice(0, 256), slice(M - 256, M)):
+        assert _rel_err(c[rows].cpu(), ok.gemm(a[rows].cpu(), b.cpu())) <= 1e-2
+
+
 def test_gemm_rejects_bad_shapes(ops):
     from lego_amd.runtime import LegoHipError
     with pytest.raises(LegoHipError):
