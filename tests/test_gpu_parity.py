@@ -97,6 +97,19 @@ def test_transpose_of_any_shape(ops, dtype, rows, cols):
     assert (buf[rows * cols:] == 7.0).all()       # nothing past the matrix was written
 
 
+def test_transpose_offsets_beyond_32_bits(ops):
+    """More than 2^32 elements: the first and the last rows and columns of the result are compared."""
+    print("transpose of more than 2^32 elements", flush=True)
+    rows, cols = 65536 + 64, 65536
+    x = torch.empty(rows, cols, device="cuda", dtype=torch.half).normal_(generator=torch.Generator(device="cuda").manual_seed(28))
+    y = ops.transpose(x)
+    assert y.shape == (cols, rows)
+    for r in (slice(0, 64), slice(rows - 64, rows)):
+        assert torch.equal(y[:, r], x[r, :].t())
+    for c in (slice(0, 64), slice(cols - 64, cols)):
+        assert torch.equal(y[c, :], x[:, c].t())
+
+
 def test_transpose_rejects_bad_arguments(ops):
     from lego_amd.runtime import LegoHipError
     with pytest.raises(ValueError):
