@@ -64,6 +64,13 @@ int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, con
                                const float* rstd, void* dx, void* dw, void* db, void* workspace,
                                unsigned long long workspace_bytes, int M, int N, void* stream);
 
+/* The same for fp32 tensors (the reference's kernels take the tensors' own type, layernorm.py:372-405);
+ * every shape takes the two passes; the workspace has its own size. */
+int lego_hip_layernorm_bwd_f32_workspace_bytes(int M, int N, unsigned long long* bytes);
+int lego_hip_layernorm_bwd_f32(const void* dy, const void* x, const void* w, const float* mean,
+                               const float* rstd, void* dx, void* dw, void* db, void* workspace,
+                               unsigned long long workspace_bytes, int M, int N, void* stream);
+
 /* C = A * B, A is M x K, B is K x N, C is M x N, fp16 with fp32 accumulation.
  * Replaces matmul(a, b) (reference: triton_generated/matmul/matmul_NTA_NTB.py:129-145).
  * M and N multiples of 8 (one 16-byte chunk of fp16; the 256 x 256 tiles may be ragged at the

@@ -160,6 +160,27 @@ int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, con
                                              as_stream(stream)));
 }
 
+int lego_hip_layernorm_bwd_f32_workspace_bytes(int M, int N, unsigned long long* bytes)
+{
+  if (bytes == nullptr || M <= 0 || N <= 0 || N > LEGO_LAYERNORM_BWD_MAX_N) return kInvalid;
+  const unsigned long long pitch = (static_cast<unsigned long long>(N) + 7) / 8 * 8;
+  *bytes = 2ull * lego_layernorm_bwd_f32_groups(M, N) * pitch * sizeof(float);
+  return 0;
+}
+
+int lego_hip_layernorm_bwd_f32(const void* dy, const void* x, const void* w, const float* mean,
+                               const float* rstd, void* dx, void* dw, void* db, void* workspace,
+                               unsigned long long workspace_bytes, int M, int N, void* stream)
+{
+  unsigned long long need = 0;
+  if (lego_hip_layernorm_bwd_f32_workspace_bytes(M, N, &need) != 0) return kInvalid;
+  if (!usable(dy) || !usable(x) || !usable(w) || !usable(dx) || !usable(dw) || !usable(db) || !usable(workspace))
+    return kInvalid;
+  if (mean == nullptr || rstd == nullptr || workspace_bytes < need) return kInvalid;
+  return ok_or(lego_layernorm_bwd_f32_launch(dy, x, w, mean, rstd, dx, dw, db, static_cast<float*>(workspace), M, N,
+                                             as_stream(stream)));
+}
+
 namespace {
 typedef hipError_t (*gemm_launcher)(const void*, const void*, void*, int, int, int, int, hipStream_t);
 struct GemmKernels {

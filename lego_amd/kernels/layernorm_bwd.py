@@ -45,9 +45,10 @@ def emit():
         row_base=code(tidy(X[row, 0, 0, 0], {row: (0, M)})).replace("row", "static_cast<size_t>(row)"),
         vecs={th: code(it * th + t) for th in sorted({th for th, _ in CONFIGS + (LONG,)})},
         vec_off=code(tidy(X[0, v, 0, 0], {v: (0, N / 8)})),
+        vec_off4=code(tidy(OrderBy(Row(M, N)).TileBy([M, N / 4], [1, 4])[0, v, 0, 0], {v: (0, N / 4)})),
         stat_off=code(OrderBy(Row(M)).TileBy([M])[row,]),
         part_off=code(tidy(P[wg, v, 0, 0], {wg: (0, G), v: (0, N / 8)})).replace("wg", "static_cast<size_t>(wg)"),
     )
     text = template("layernorm_bwd.hip.j2").render(**params)
-    return Emitted("layernorm_bwd_f16.hip", text, ["lego_layernorm_bwd_f16_launch"]), dict(
+    return Emitted("layernorm_bwd_f16.hip", text, ["lego_layernorm_bwd_f16_launch", "lego_layernorm_bwd_f32_launch"]), dict(
         MAX_N=LONG[0] * LONG[1] * 8, MAX_GROUPS=MAX_GROUPS)

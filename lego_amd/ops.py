@@ -105,22 +105,25 @@ def layer_norm_fwd(x, weight, bias, eps=1e-5, waves_per_row: int | None = None):
 
 
 def layer_norm_bwd(dy, x, weight, mean, rstd):
-    """LayerNorm backward; returns ``(dx, dw, db)``.  fp16, rows of up to 32768 elements."""
+    """LayerNorm backward; returns ``(dx, dw, db)``.  fp16 or fp32 tensors, rows of up to 32768 elements."""
+    if x.dtype not in (torch.float16, torch.float32):
+        raise ValueError("x must be float16 or float32")
+    tag = "f16" if x.dtype == torch.float16 else "f32"
     x_arg = x.reshape(-1, x.shape[-1])
-    dy_arg = dy.reshape(-1, dy.shape[-1])
-    _check(x_arg, torch.float16, "x")
-    _check(dy_arg.contiguous(), torch.float16, "dy")
-    dy_arg = dy_arg.contiguous()
-    _check(weight, torch.float16, "weight", ndim=1)
+    dy_arg = dy.reshape(-1, dy.shape[-1]).contiguous()
+    _check(x_arg, x.dtype, "x")
+    _check(dy_arg, x.dtype, "dy")
+    _check(weight, x.dtype, "weight", ndim=1)
     M, N = x_arg.shape
     need = ctypes.c_ulonglong(0)
-    runtime.call("lego_hip_layernorm_bwd_workspace_bytes", M, N, ctypes.byref(need))
+    runtime.call("lego_hip_layernorm_bwd_workspace_bytes" if tag == "f16" else "lego_hip_layernorm_bwd_f32_workspace_bytes",
+                 M, N, ctypes.byref(need))
     # like the reference's wrapper, which allocates its partial buffers with torch (layernorm.py:381-383)
     workspace = torch.empty(need.value // 4, dtype=torch.float32, device=x.device)
     dx = torch.empty_like(x_arg)
     dw = torch.empty((N,), dtype=weight.dtype, device=x.device)
     db = torch.empty((N,), dtype=weight.dtype, device=x.device)
-    runtime.call("lego_hip_layernorm_bwd_f16", _ptr(dy_arg), _ptr(x_arg), _ptr(weight), _ptr(mean), _ptr(rstd),
+    runtime.call(f"lego_hip_layernorm_bwd_{tag}", _ptr(dy_arg), _ptr(x_arg), _ptr(weight), _ptr(mean), _ptr(rstd),
                  _ptr(dx), _ptr(dw), _ptr(db), _ptr(workspace), need, M, N, _stream())
     return dx.view(x.shape), dw, db
 

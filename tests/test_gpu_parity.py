@@ -307,6 +307,25 @@ def test_layernorm_backward_matches_oracle(ops, M, N):
     assert (db.cpu().float() - bc.grad).abs().max().item() <= 2e-3 * max(1.0, bc.grad.abs().max().item())
 
 
+@pytest.mark.parametrize("M,N", [(1, 4), (7, 5), (300, 1000), (129, 4096), (33, 4099), (40, 16384)])
+def test_layernorm_backward_fp32(ops, M, N):
+    """fp32 tensors through the autograd wrapper, against fp64 autograd on the CPU."""
+    from lego_amd.ops import lego_layer_norm
+    print(f"layernorm backward fp32 {M}x{N}", flush=True)
+    g = _gen(29)
+    x = 2.0 * torch.randn(M, N, generator=g)
+    w = 1 + 0.1 * torch.randn(N, generator=g)
+    b = 0.1 * torch.randn(N, generator=g)
+    dy = 0.1 * torch.randn(M, N, generator=g)
+    xd, wd, bd = (t.cuda().requires_grad_(True) for t in (x, w, b))
+    lego_layer_norm(xd, (N,), wd, bd, 1e-5).backward(dy.cuda())
+    xc, wc, bc = (t.double().requires_grad_(True) for t in (x, w, b))
+    torch.nn.functional.layer_norm(xc, (N,), wc, bc, 1e-5).backward(dy.double())
+    assert (xd.grad.cpu().double() - xc.grad).abs().max().item() <= 2e-5
+    assert (wd.grad.cpu().double() - wc.grad).abs().max().item() <= 2e-5 * max(1.0, wc.grad.abs().max().item())
+    assert (bd.grad.cpu().double() - bc.grad).abs().max().item() <= 2e-5 * max(1.0, bc.grad.abs().max().item())
+
+
 def test_config3_full_size(ops):
     print("config 3 full size", flush=True)
     g = _gen(2)
