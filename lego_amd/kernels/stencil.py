@@ -57,11 +57,15 @@ def emit():
     H, h, hx, hy = size("H"), idx("h"), idx("hx"), idx("hy")
     shell_rows = OrderBy(Row(H, H)).TileBy([H, H])
     shell_inv = [code(tidy(e, {h: (0, H * H)})) for e in shell_rows.inv(h)]
-    shell = OrderBy(Row(H, H, ROW_WORDS)).TileBy([H, H, ROW_WORDS])
-    shell_row = code(tidy(shell[hx, hy, 0], {hx: (0, H), hy: (0, H)}))
+    # rows hy of one hx are ROW_WORDS apart, the planes hx are PLANE >= H*ROW_WORDS words apart (padded so that
+    # the sixteen lanes of one 16-byte access, rows (i, 0..7) and (i+1, 0..7), fall into sixteen different
+    # groups of four banks: see the kernel source)
+    PLANE = size("PLANE")
+    shell = OrderBy(Row(H, PLANE)).TileBy([H, PLANE])
+    shell_row = code(tidy(shell[hx, ROW_WORDS * hy], {hx: (0, H), hy: (0, H)}))
     params = dict(
-        shell_layout=f"OrderBy(Row(H, H, {ROW_WORDS})).TileBy([H, H, {ROW_WORDS}])[hx, hy, word]",
-        shell_inv=shell_inv, shell_row=shell_row, ROW_WORDS=ROW_WORDS,
+        shell_layout=f"OrderBy(Row(H, PLANE)).TileBy([H, PLANE])[hx, {ROW_WORDS}*hy + word]",
+        shell_inv=shell_inv, shell_row=shell_row, ROW_WORDS=ROW_WORDS, UNPADDED_RADIUS=2,
         banner=BANNER, B=B, MAX_RADIUS=MAX_RADIUS, WAVES=WAVES,
         row_layout=f"Row({B}, {B})",
         normal_layout=f"OrderBy(Row(N, N, N)).TileBy([N/{B}]*3, [{B}]*3)[x/{B}, y/{B}, z/{B}, x%{B}, y%{B}, z%{B}]",
