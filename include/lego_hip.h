@@ -41,8 +41,11 @@ int lego_hip_transpose_f16(const void* in, void* out, int rows, int cols, void* 
 int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream);
 int lego_hip_softmax_f32(const void* x, void* y, int M, int N, void* stream);
 
+/* The same for bfloat16 tensors (the reference's kernel takes the tensor's own type, softmax.py:97-160). */
+int lego_hip_softmax_bf16(const void* x, void* y, int M, int N, void* stream);
+
 /* LayerNorm forward over the last dimension of an M x N matrix; x, y, w, b share one element
- * type (fp16 or fp32), w and b have N elements; mean, rstd are fp32 [M] outputs.  Replaces
+ * type (fp16, bfloat16 or fp32), w and b have N elements; mean, rstd are fp32 [M] outputs.  Replaces
  * LEGOLayerNorm.forward / lego_layer_norm (reference:
  * triton_generated/layernorm/layernorm.py:279-307, whose limit is 64 KiB of row, :291-294).
  * Any N up to 32768. */
@@ -50,6 +53,8 @@ int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void
                                float* mean, float* rstd, int M, int N, float eps, void* stream);
 int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void* b,
                                float* mean, float* rstd, int M, int N, float eps, void* stream);
+int lego_hip_layernorm_fwd_bf16(const void* x, void* y, const void* w, const void* b,
+                                float* mean, float* rstd, int M, int N, float eps, void* stream);
 
 /* LayerNorm backward: dx (M x N fp16), dw and db (N fp16) from dy, x, w and the forward pass's
  * mean and rstd.  Replaces LEGOLayerNorm.backward (reference:
@@ -70,6 +75,11 @@ int lego_hip_layernorm_bwd_f32_workspace_bytes(int M, int N, unsigned long long*
 int lego_hip_layernorm_bwd_f32(const void* dy, const void* x, const void* w, const float* mean,
                                const float* rstd, void* dx, void* dw, void* db, void* workspace,
                                unsigned long long workspace_bytes, int M, int N, void* stream);
+/* ... and for bfloat16 tensors. */
+int lego_hip_layernorm_bwd_bf16_workspace_bytes(int M, int N, unsigned long long* bytes);
+int lego_hip_layernorm_bwd_bf16(const void* dy, const void* x, const void* w, const float* mean,
+                                const float* rstd, void* dx, void* dw, void* db, void* workspace,
+                                unsigned long long workspace_bytes, int M, int N, void* stream);
 
 /* C = A * B, A is M x K, B is K x N, C is M x N, fp16 with fp32 accumulation.
  * Replaces matmul(a, b) (reference: triton_generated/matmul/matmul_NTA_NTB.py:129-145).

@@ -41,7 +41,9 @@ TRANSPOSE = {
 # element-per-access kernels ("s") take any N
 ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f32", True, 1), ("f32", True, 4),
            ("f16", False, 1), ("f32", False, 1), ("f16", False, 4), ("f32", False, 4),
-           ("f16", True, 16), ("f32", True, 16), ("f16", False, 16), ("f32", False, 16)]
+           ("f16", True, 16), ("f32", True, 16), ("f16", False, 16), ("f32", False, 16),
+           ("bf16", True, 1), ("bf16", True, 4), ("bf16", True, 16), ("bf16", False, 1), ("bf16", False, 4),
+           ("bf16", False, 16)]
 ROWWISE_DEFAULT_WAVES = 4
 ROWWISE_MAX_N = rowwise.MAX_N
 GEMM = dict(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8)
@@ -113,8 +115,8 @@ def generate():
         h += [f"hipError_t lego_softmax_{tag}_w{w}_launch(const void*, void*, int, int, hipStream_t);",
               f"hipError_t lego_layernorm_fwd_{tag}_w{w}_launch(const void*, void*, const void*, const void*, "
               "float*, float*, int, int, float, hipStream_t);"]
-    h += ["hipError_t lego_softmax_long_f16_launch(const void*, void*, int, int, hipStream_t);",
-          "hipError_t lego_softmax_long_f32_launch(const void*, void*, int, int, hipStream_t);",
+    h += [f"hipError_t lego_softmax_long_{d}_launch(const void*, void*, int, int, hipStream_t);" for d in rowwise.ELEMENTS]
+    h += [
           f"#define LEGO_ROWWISE_MAX_N {ROWWISE_MAX_N}",
           f"#define LEGO_ROWWISE_MAX_N_SMALL_TEAMS {rowwise.MAX_N_SMALL_TEAMS}",
           "// waves per row: one wave keeps short rows free of barriers, four waves keep the",
@@ -123,7 +125,10 @@ def generate():
           f"inline int lego_rowwise_default_wpr(int n) {{ return n <= 2048 ? 1 : n <= {rowwise.MAX_N_SMALL_TEAMS} ? "
           f"{ROWWISE_DEFAULT_WAVES} : {rowwise.LONG_ROW_WAVES}; }}", ""]
     h += ["unsigned lego_layernorm_bwd_groups(int M, int N);", "unsigned lego_layernorm_bwd_f32_groups(int M, int N);",
+          "unsigned lego_layernorm_bwd_bf16_groups(int M, int N);",
           "hipError_t lego_layernorm_bwd_f32_launch(const void*, const void*, const void*, const float*, const float*, "
+          "void*, void*, void*, float*, int, int, hipStream_t);",
+          "hipError_t lego_layernorm_bwd_bf16_launch(const void*, const void*, const void*, const float*, const float*, "
           "void*, void*, void*, float*, int, int, hipStream_t);",
           "hipError_t lego_layernorm_bwd_f16_launch(const void*, const void*, const void*, const float*, const float*, "
           "void*, void*, void*, float*, int, int, hipStream_t);",

@@ -139,6 +139,33 @@ int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void
       x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
 }
 
+int lego_hip_softmax_bf16(const void* x, void* y, int M, int N, void* stream)
+{
+  if (!usable(x) || !usable(y) || M <= 0 || N <= 0) return kInvalid;
+  if (N > LEGO_ROWWISE_MAX_N) return ok_or(lego_softmax_long_bf16_launch(x, y, M, N, as_stream(stream)));   // two passes
+  const int wpr = lego_rowwise_default_wpr(N);
+  if (N % 8)   // ragged rows
+    return ok_or((wpr == 16 ? lego_softmax_bf16s_w16_launch : wpr == 1 ? lego_softmax_bf16s_w1_launch
+                                                                       : lego_softmax_bf16s_w4_launch)(x, y, M, N, as_stream(stream)));
+  return ok_or((wpr == 16 ? lego_softmax_bf16_w16_launch : wpr == 1 ? lego_softmax_bf16_w1_launch
+                                                                    : lego_softmax_bf16_w4_launch)(x, y, M, N, as_stream(stream)));
+}
+
+int lego_hip_layernorm_fwd_bf16(const void* x, void* y, const void* w, const void* b,
+                                float* mean, float* rstd, int M, int N, float eps, void* stream)
+{
+  if (!usable(x) || !usable(y) || !usable(w) || !usable(b) || mean == nullptr || rstd == nullptr) return kInvalid;
+  if (M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
+  const int wpr = lego_rowwise_default_wpr(N);
+  if (N % 8)   // ragged rows
+    return ok_or((wpr == 16 ? lego_layernorm_fwd_bf16s_w16_launch : wpr == 1 ? lego_layernorm_fwd_bf16s_w1_launch
+                                                                             : lego_layernorm_fwd_bf16s_w4_launch)(
+        x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+  return ok_or((wpr == 16 ? lego_layernorm_fwd_bf16_w16_launch : wpr == 1 ? lego_layernorm_fwd_bf16_w1_launch
+                                                                          : lego_layernorm_fwd_bf16_w4_launch)(
+      x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+}
+
 int lego_hip_layernorm_bwd_workspace_bytes(int M, int N, unsigned long long* bytes)
 {
   if (bytes == nullptr || M <= 0 || N <= 0 || N > LEGO_LAYERNORM_BWD_MAX_N) return kInvalid;
@@ -179,6 +206,27 @@ int lego_hip_layernorm_bwd_f32(const void* dy, const void* x, const void* w, con
   if (mean == nullptr || rstd == nullptr || workspace_bytes < need) return kInvalid;
   return ok_or(lego_layernorm_bwd_f32_launch(dy, x, w, mean, rstd, dx, dw, db, static_cast<float*>(workspace), M, N,
                                              as_stream(stream)));
+}
+
+int lego_hip_layernorm_bwd_bf16_workspace_bytes(int M, int N, unsigned long long* bytes)
+{
+  if (bytes == nullptr || M <= 0 || N <= 0 || N > LEGO_LAYERNORM_BWD_MAX_N) return kInvalid;
+  const unsigned long long pitch = (static_cast<unsigned long long>(N) + 7) / 8 * 8;
+  *bytes = 2ull * lego_layernorm_bwd_bf16_groups(M, N) * pitch * sizeof(float);
+  return 0;
+}
+
+int lego_hip_layernorm_bwd_bf16(const void* dy, const void* x, const void* w, const float* mean,
+                                const float* rstd, void* dx, void* dw, void* db, void* workspace,
+                                unsigned long long workspace_bytes, int M, int N, void* stream)
+{
+  unsigned long long need = 0;
+  if (lego_hip_layernorm_bwd_bf16_workspace_bytes(M, N, &need) != 0) return kInvalid;
+  if (!usable(dy) || !usable(x) || !usable(w) || !usable(dx) || !usable(dw) || !usable(db) || !usable(workspace))
+    return kInvalid;
+  if (mean == nullptr || rstd == nullptr || workspace_bytes < need) return kInvalid;
+  return ok_or(lego_layernorm_bwd_bf16_launch(dy, x, w, mean, rstd, dx, dw, db, static_cast<float*>(workspace), M, N,
+                                              as_stream(stream)));
 }
 
 namespace {

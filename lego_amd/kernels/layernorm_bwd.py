@@ -50,5 +50,5 @@ def emit():
         part_off=code(tidy(P[wg, v, 0, 0], {wg: (0, G), v: (0, N / 8)})).replace("wg", "static_cast<size_t>(wg)"),
     )
     text = template("layernorm_bwd.hip.j2").render(**params)
-    return Emitted("layernorm_bwd_f16.hip", text, ["lego_layernorm_bwd_f16_launch", "lego_layernorm_bwd_f32_launch"]), dict(
+    return Emitted("layernorm_bwd_f16.hip", text, ["lego_layernorm_bwd_f16_launch", "lego_layernorm_bwd_f32_launch", "lego_layernorm_bwd_bf16_launch"]), dict(
         MAX_N=LONG[0] * LONG[1] * 8, MAX_GROUPS=MAX_GROUPS)

@@ -19,6 +19,7 @@ from __future__ import annotations
 from ..lego import OrderBy, Row
 from .common import BANNER, Emitted, code, idx, size, template, tidy
 
+ELEMENTS = {"f16": ("_Float16", 2), "bf16": ("__bf16", 2), "f32": ("float", 4)}
 THREADS = 256                  # lanes per workgroup; a team of 16 waves is a workgroup of 1024
 MAX_N = 32768                  # the reference's fp16 LayerNorm limit (64 KiB of row, layernorm_triton.py:335-338)
 MAX_N_SMALL_TEAMS = 16384      # teams of up to four waves; longer rows take sixteen
@@ -32,7 +33,7 @@ def emit(waves_per_row=1, dtype="f16", vectorised=True):
     and alignment (the reference's own softmax test is 1823 x 781): the elements before a row's
     first 16-byte boundary and after its last whole vector go one per lane, the rest as vectors."""
     WPR = waves_per_row
-    elt, esize = {"f16": ("_Float16", 2), "f32": ("float", 4)}[dtype]
+    elt, esize = ELEMENTS[dtype]
     EPV = 16 // esize
     tag = dtype if vectorised else dtype + "s"
     TEAM = 64 * WPR
@@ -78,7 +79,7 @@ def emit_long():
     M, N = size("M"), size("N")
     row, v = idx("row"), idx("v")
     variants, vec_off = [], {}
-    for dtype, (elt, esize) in (("f16", ("_Float16", 2)), ("f32", ("float", 4))):
+    for dtype, (elt, esize) in ELEMENTS.items():
         epv = 16 // esize
         variants.append((dtype, elt, epv))
         X = OrderBy(Row(M, N)).TileBy([M, N / epv], [1, epv])
@@ -88,4 +89,4 @@ def emit_long():
         banner=BANNER, THREADS=1024, VARIANTS=variants, vec_off=vec_off,
         row_base=code(row_base).replace("row", "static_cast<size_t>(row)"),
         x_layout="OrderBy(Row(M, N)).TileBy([M, N/EPV], [1, EPV])[row, v, 0, :]")
-    return Emitted("softmax_long.hip", text, ["lego_softmax_long_f16_launch", "lego_softmax_long_f32_launch"])
+    return Emitted("softmax_long.hip", text, [f"lego_softmax_long_{d}_launch" for d in ELEMENTS])

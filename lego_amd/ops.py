@@ -59,19 +59,20 @@ def transpose(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
+_ROW_TAG = {torch.float16: "f16", torch.bfloat16: "bf16", torch.float32: "f32"}
+
+
 def softmax(x: torch.Tensor, waves_per_row: int | None = None) -> torch.Tensor:
-    """Row softmax of a 2-D fp16 or fp32 tensor."""
-    if x.dtype not in (torch.float16, torch.float32):
-        raise ValueError("softmax supports float16 and float32")
+    """Row softmax of a 2-D fp16, bf16 or fp32 tensor."""
+    if x.dtype not in _ROW_TAG:
+        raise ValueError("softmax supports float16, bfloat16 and float32")
     _check(x, x.dtype, "x")
     n_rows, n_cols = x.shape
     y = torch.empty_like(x)
-    if x.dtype == torch.float32:
-        if waves_per_row is not None:
-            raise ValueError("waves_per_row is a tuning knob of the fp16 kernels")
-        runtime.call("lego_hip_softmax_f32", _ptr(x), _ptr(y), n_rows, n_cols, _stream())
-    elif waves_per_row is None:
-        runtime.call("lego_hip_softmax_f16", _ptr(x), _ptr(y), n_rows, n_cols, _stream())
+    if waves_per_row is None:
+        runtime.call(f"lego_hip_softmax_{_ROW_TAG[x.dtype]}", _ptr(x), _ptr(y), n_rows, n_cols, _stream())
+    elif x.dtype != torch.float16:
+        raise ValueError("waves_per_row is a tuning knob of the fp16 kernels")
     else:
         runtime.call("lego_hip_softmax_f16_wpr", _ptr(x), _ptr(y), n_rows, n_cols, waves_per_row, _stream())
     return y
@@ -79,8 +80,8 @@ def softmax(x: torch.Tensor, waves_per_row: int | None = None) -> torch.Tensor:
 
 def layer_norm_fwd(x, weight, bias, eps=1e-5, waves_per_row: int | None = None):
     """LayerNorm forward over the last dimension; returns ``(y, mean, rstd)``."""
-    if x.dtype not in (torch.float16, torch.float32):
-        raise ValueError("x must be float16 or float32")
+    if x.dtype not in _ROW_TAG:
+        raise ValueError("x must be float16, bfloat16 or float32")
     x_arg = x.reshape(-1, x.shape[-1])
     _check(x_arg, x.dtype, "x")
     M, N = x_arg.shape
@@ -95,20 +96,20 @@ def layer_norm_fwd(x, weight, bias, eps=1e-5, waves_per_row: int | None = None):
     mean = torch.empty((M,), dtype=torch.float32, device=x.device)
     rstd = torch.empty((M,), dtype=torch.float32, device=x.device)
     args = (_ptr(x_arg), _ptr(y), _ptr(weight), _ptr(bias), _ptr(mean), _ptr(rstd), M, N, float(eps))
-    if x.dtype == torch.float32:
-        runtime.call("lego_hip_layernorm_fwd_f32", *args, _stream())
-    elif waves_per_row is None:
-        runtime.call("lego_hip_layernorm_fwd_f16", *args, _stream())
+    if waves_per_row is None:
+        runtime.call(f"lego_hip_layernorm_fwd_{_ROW_TAG[x.dtype]}", *args, _stream())
+    elif x.dtype != torch.float16:
+        raise ValueError("waves_per_row is a tuning knob of the fp16 kernels")
     else:
         runtime.call("lego_hip_layernorm_fwd_f16_wpr", *args, waves_per_row, _stream())
     return y.view(x.shape), mean, rstd
 
 
 def layer_norm_bwd(dy, x, weight, mean, rstd):
-    """LayerNorm backward; returns ``(dx, dw, db)``.  fp16 or fp32 tensors, rows of up to 32768 elements."""
-    if x.dtype not in (torch.float16, torch.float32):
-        raise ValueError("x must be float16 or float32")
-    tag = "f16" if x.dtype == torch.float16 else "f32"
+    """LayerNorm backward; returns ``(dx, dw, db)``.  fp16, bf16 or fp32 tensors, rows of up to 32768 elements."""
+    if x.dtype not in _ROW_TAG:
+        raise ValueError("x must be float16, bfloat16 or float32")
+    tag = _ROW_TAG[x.dtype]
     x_arg = x.reshape(-1, x.shape[-1])
     dy_arg = dy.reshape(-1, dy.shape[-1]).contiguous()
     _check(x_arg, x.dtype, "x")
@@ -116,7 +117,7 @@ def layer_norm_bwd(dy, x, weight, mean, rstd):
     _check(weight, x.dtype, "weight", ndim=1)
     M, N = x_arg.shape
     need = ctypes.c_ulonglong(0)
-    runtime.call("lego_hip_layernorm_bwd_workspace_bytes" if tag == "f16" else "lego_hip_layernorm_bwd_f32_workspace_bytes",
+    runtime.call("lego_hip_layernorm_bwd_workspace_bytes" if tag == "f16" else f"lego_hip_layernorm_bwd_{tag}_workspace_bytes",
                  M, N, ctypes.byref(need))
     # like the reference's wrapper, which allocates its partial buffers with torch (layernorm.py:381-383)
     workspace = torch.empty(need.value // 4, dtype=torch.float32, device=x.device)

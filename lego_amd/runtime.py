@@ -22,8 +22,11 @@ SIGNATURES = {
     "lego_hip_transpose_f16": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "lego_hip_softmax_f16": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "lego_hip_softmax_f32": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+    "lego_hip_softmax_bf16": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "lego_hip_layernorm_fwd_f32": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                    _c_int, _c_int, _c_float, _c_void_p],
+    "lego_hip_layernorm_fwd_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                                    _c_int, _c_int, _c_float, _c_void_p],
     "lego_hip_layernorm_fwd_f16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                    _c_int, _c_int, _c_float, _c_void_p],
     "lego_hip_gemm_f16": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
@@ -46,6 +49,8 @@ SIGNATURES = {
     "lego_hip_layernorm_bwd_f16": [_c_void_p] * 9 + [ctypes.c_ulonglong, _c_int, _c_int, _c_void_p],
     "lego_hip_layernorm_bwd_f32_workspace_bytes": [_c_int, _c_int, ctypes.POINTER(ctypes.c_ulonglong)],
     "lego_hip_layernorm_bwd_f32": [_c_void_p] * 9 + [ctypes.c_ulonglong, _c_int, _c_int, _c_void_p],
+    "lego_hip_layernorm_bwd_bf16_workspace_bytes": [_c_int, _c_int, ctypes.POINTER(ctypes.c_ulonglong)],
+    "lego_hip_layernorm_bwd_bf16": [_c_void_p] * 9 + [ctypes.c_ulonglong, _c_int, _c_int, _c_void_p],
     "lego_hip_copy16": [_c_void_p, _c_void_p, ctypes.c_ulonglong, _c_void_p],
     "lego_hip_copy16_stream": [_c_void_p, _c_void_p, ctypes.c_ulonglong, _c_void_p],
 }

@@ -326,6 +326,40 @@ def test_layernorm_backward_fp32(ops, M, N):
     assert (bd.grad.cpu().double() - bc.grad).abs().max().item() <= 2e-5 * max(1.0, bc.grad.abs().max().item())
 
 
+@pytest.mark.parametrize("M,N", [(5, 8), (9, 781), (33, 2048), (64, 8192), (3, 8191), (4, 20000), (2, 32768), (2, 50257)])
+def test_softmax_bfloat16(ops, M, N):
+    print(f"softmax bf16 {M}x{N}", flush=True)
+    x = (2.0 * torch.randn(M, N, generator=_gen(30))).bfloat16()
+    want = torch.softmax(x.float(), -1)
+    got = ops.softmax(x.cuda()).cpu()
+    assert got.dtype == torch.bfloat16
+    # half a bfloat16 spacing of the largest possible value, 1: 2^-9
+    assert (got.float() - want).abs().max().item() <= 2.0 ** -9 + 1e-6
+
+
+@pytest.mark.parametrize("M,N", [(5, 8), (9, 781), (33, 2048), (64, 8192), (3, 8191), (4, 20000), (2, 32768)])
+def test_layernorm_bfloat16_forward_and_backward(ops, M, N):
+    """bfloat16 tensors through the autograd wrapper, against fp32 autograd on the CPU."""
+    from lego_amd.ops import lego_layer_norm
+    print(f"layernorm bf16 {M}x{N}", flush=True)
+    g = _gen(31)
+    x = (2.0 * torch.randn(M, N, generator=g)).bfloat16()
+    w = (1 + 0.1 * torch.randn(N, generator=g)).bfloat16()
+    b = (0.1 * torch.randn(N, generator=g)).bfloat16()
+    dy = (0.1 * torch.randn(M, N, generator=g)).bfloat16()
+    xd, wd, bd = (t.cuda().requires_grad_(True) for t in (x, w, b))
+    y = lego_layer_norm(xd, (N,), wd, bd, 1e-5)
+    y.backward(dy.cuda())
+    xc, wc, bc = (t.float().requires_grad_(True) for t in (x, w, b))
+    yr = torch.nn.functional.layer_norm(xc, (N,), wc, bc, 1e-5)
+    yr.backward(dy.float())
+    # results are rounded to bfloat16: half a spacing relative to the magnitude, 2^-9
+    assert ((y.detach().cpu().float() - yr.detach()).abs() <= 2.0 ** -8 * yr.detach().abs() + 1e-3).all()
+    assert ((xd.grad.cpu().float() - xc.grad).abs() <= 2.0 ** -8 * xc.grad.abs() + 1e-3).all()
+    assert ((wd.grad.cpu().float() - wc.grad).abs() <= 2.0 ** -8 * wc.grad.abs() + 2e-3 * max(1.0, wc.grad.abs().max().item())).all()
+    assert ((bd.grad.cpu().float() - bc.grad).abs() <= 2.0 ** -8 * bc.grad.abs() + 2e-3 * max(1.0, bc.grad.abs().max().item())).all()
+
+
 def test_config3_full_size(ops):
     print("config 3 full size", flush=True)
     g = _gen(2)
