@@ -71,3 +71,19 @@ def test_gpu_rejects_bad_sizes():
     from lego_amd.runtime import LegoHipError
     with pytest.raises(LegoHipError):
         ops.lud(torch.eye(100, device="cuda"))
+
+
+@pytest.mark.gpu
+def test_gpu_large_matrix_reproduces_its_factors():
+    """n = 16384, the size the reference publishes: L*U gives the matrix back (fp32, diagonally dominant)."""
+    from lego_amd import ops
+    print("lud n=16384", flush=True)
+    n = 16384
+    a = torch.rand(n, n, device="cuda", generator=torch.Generator(device="cuda").manual_seed(61))
+    a.diagonal().add_(float(n))
+    w = a.clone()
+    ops.lud(w)
+    lower = torch.tril(w, -1)
+    lower.diagonal().fill_(1.0)
+    back = lower @ torch.triu(w)
+    assert ((back - a).norm() / a.norm()).item() <= 1e-5

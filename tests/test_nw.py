@@ -87,3 +87,22 @@ def test_gpu_rejects_bad_sizes():
     with pytest.raises(LegoHipError):
         ops.needleman_wunsch(torch.zeros(101, 101, dtype=torch.int32, device="cuda"),
                              torch.zeros(101, 101, dtype=torch.int32, device="cuda"), 10)
+
+
+@pytest.mark.gpu
+def test_gpu_maximum_size_closed_form():
+    """The largest size the entry point takes, n = 32768: with zero scores a diagonal step is free and a
+    gap costs the penalty, so m[i][j] = -|i - j| * penalty."""
+    from lego_amd import ops
+    print("needleman-wunsch n=32768, zero scores", flush=True)
+    n, penalty = 32768, 3
+    ref = torch.zeros((n + 1, n + 1), dtype=torch.int32, device="cuda")
+    m = torch.zeros((n + 1, n + 1), dtype=torch.int32, device="cuda")
+    border = -torch.arange(n + 1, dtype=torch.int32, device="cuda") * penalty
+    m[0, :] = border
+    m[:, 0] = border
+    ops.needleman_wunsch(ref, m, penalty)
+    idx = torch.arange(n + 1, device="cuda", dtype=torch.int32)
+    for rows in (slice(0, 130), slice(16000, 16130), slice(n - 129, n + 1)):
+        want = -(idx[rows, None] - idx[None, :]).abs() * penalty
+        assert torch.equal(m[rows], want)
