@@ -36,6 +36,19 @@ WAVES = 4             # bricks per workgroup
 ROW_WORDS = 20
 
 
+UNPADDED_RADIUS = 2    # its padding would cost the third workgroup per CU, which is worth more (measured)
+
+
+def shell_plane(radius):
+    """Words between the planes ``hx`` of the shell in LDS.  A 16-byte access of 64 lanes is served 16
+    lanes at a time, rows ``(i, 0..7)`` and ``(i+1, 0..7)`` of the shell: with rows ``ROW_WORDS`` = 20
+    words apart the eight rows of one plane start in eight different groups of four banks
+    (``5*j mod 16``), and the padding puts the next plane eight groups further, on the other eight."""
+    h, g = B + 2 * radius, ROW_WORDS // 4
+    pad = 0 if radius == UNPADDED_RADIUS else 4 * ((8 - g * h) % 16)
+    return h * ROW_WORDS + pad
+
+
 def layouts(nb):
     """``(row-major, bricks)`` layouts of a cube of ``nb`` bricks per side."""
     levels = ([nb, nb, nb], [B, B, B])
@@ -65,7 +78,8 @@ def emit():
     shell_row = code(tidy(shell[hx, ROW_WORDS * hy], {hx: (0, H), hy: (0, H)}))
     params = dict(
         shell_layout=f"OrderBy(Row(H, PLANE)).TileBy([H, PLANE])[hx, {ROW_WORDS}*hy + word]",
-        shell_inv=shell_inv, shell_row=shell_row, ROW_WORDS=ROW_WORDS, UNPADDED_RADIUS=2,
+        shell_inv=shell_inv, shell_row=shell_row, ROW_WORDS=ROW_WORDS,
+        PLANES={B + 2 * r: shell_plane(r) for r in range(1, MAX_RADIUS + 1)},
         banner=BANNER, B=B, MAX_RADIUS=MAX_RADIUS, WAVES=WAVES,
         row_layout=f"Row({B}, {B})",
         normal_layout=f"OrderBy(Row(N, N, N)).TileBy([N/{B}]*3, [{B}]*3)[x/{B}, y/{B}, z/{B}, x%{B}, y%{B}, z%{B}]",

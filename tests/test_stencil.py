@@ -70,6 +70,28 @@ def test_bricks_order_matches_the_reference_offsets():
     assert sorted(small.ravel().tolist()) == list(range(16 ** 3))
 
 
+def test_shell_rows_in_lds_spread_over_the_banks():
+    """The sixteen lanes that a 16-byte LDS access serves together read rows (i, 0..7) and (i+1, 0..7) of the
+    shell: with 20-word rows and the padded planes of the kernel they start in sixteen different groups of
+    four banks, for every neighbour offset (radius 1 and 3; the radius-2 shell is left unpadded on purpose)."""
+    from lego_amd.kernels import stencil
+    words = stencil.ROW_WORDS
+    for radius in (1, 3):
+        h = 8 + 2 * radius
+        plane = stencil.shell_plane(radius)
+        assert plane % 4 == 0 and plane >= h * words
+        for di in range(-radius, radius + 1):
+            for dj in range(-radius, radius + 1):
+                for first in range(0, 64, 16):
+                    groups = set()
+                    for lane in range(first, first + 16):
+                        i, j = divmod(lane, 8)
+                        word = plane * (i + radius + di) + words * (j + radius + dj)
+                        assert word % 4 == 0
+                        groups.add((word // 4) % 16)
+                    assert len(groups) == 16
+
+
 def _to_bricks(x, order):
     out = torch.empty(x.numel(), dtype=x.dtype)
     out[torch.from_numpy(order).reshape(-1)] = x.reshape(-1)
