@@ -76,7 +76,12 @@ def emit():
     PLANE = size("PLANE")
     shell = OrderBy(Row(H, PLANE)).TileBy([H, PLANE])
     shell_row = code(tidy(shell[hx, ROW_WORDS * hy], {hx: (0, H), hy: (0, H)}))
+    # the star stencil exchanges only the B points of a row: planes of B*H + 4 words
+    SPLANE = size("PLANE")
+    star = OrderBy(Row(H, SPLANE)).TileBy([H, SPLANE])
+    star_row = code(tidy(star[hx, B * hy], {hx: (0, H), hy: (0, H)}))
     params = dict(
+        star_layout=f"OrderBy(Row(H, PLANE)).TileBy([H, PLANE])[hx, {B}*hy + word]", star_row=star_row,
         shell_layout=f"OrderBy(Row(H, PLANE)).TileBy([H, PLANE])[hx, {ROW_WORDS}*hy + word]",
         shell_inv=shell_inv, shell_row=shell_row, ROW_WORDS=ROW_WORDS,
         PLANES={B + 2 * r: shell_plane(r) for r in range(1, MAX_RADIUS + 1)},

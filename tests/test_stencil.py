@@ -90,6 +90,14 @@ def test_shell_rows_in_lds_spread_over_the_banks():
                         assert word % 4 == 0
                         groups.add((word // 4) % 16)
                     assert len(groups) == 16
+    # the star kernel's rows of eight words in planes of 8*H + 4 words
+    for radius in (1, 2, 3):
+        h = 8 + 2 * radius
+        plane = 8 * h + 4
+        for first in range(0, 64, 16):
+            for di, dj in ((0, 0), (radius, 0), (-radius, 0), (0, radius), (0, -radius)):
+                groups = {(plane * (lane // 8 + radius + di) + 8 * (lane % 8 + radius + dj)) // 4 % 16 for lane in range(first, first + 16)}
+                assert len(groups) == 16
 
 
 def _to_bricks(x, order):
