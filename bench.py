@@ -333,7 +333,7 @@ def main():
         ms = timed(luf, steps=2, warmup=1) - timed(lambda: wk.copy_(a0), steps=2, warmup=1)
         kernels["next_lud_f32_16384"] = dict(ms=ms, tflops=(2 / 3) * nl ** 3 / ms / 1e9,
                                              reference_ms_a100=653.5,
-                                             note="time of a matrix copy subtracted; 256 block steps of three launches")
+                                             note="time of a matrix copy subtracted; 255 block steps of two launches")
         del a0, wk
 
     # ---- CPU baseline: the oracle on a bounded panel of the headline matrix ------------------------------
