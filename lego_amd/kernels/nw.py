@@ -47,13 +47,19 @@ def emit():
     # cell (ty, tx) of block (by, bx); row 0 and column 0 of the matrices are the borders
     full = OrderBy(Row(cols, cols)).TileBy([cols, cols])
     cell = tidy(full[by * B + 1 + ty, bx * B + 1 + tx], {ty: (0, B), tx: (0, B)})
+    # The lane's share of the offset, apart: what is left is the same for all lanes of a tile row, so
+    # the accesses take a scalar base and one lane offset instead of 64-bit lane arithmetic per row.
+    cell_row = tidy(cell.subs(tx, 0), {ty: (0, B)})
+    cell_lane = sp.expand(cell - cell_row)
+    if cell_lane.free_symbols - {tx}:
+        raise ValueError(f"cell offset {cell} does not split into a row part and a lane part")
     i, j = sp.symbols("i j", integer=True, nonnegative=True)
     lds = sp.simplify(rotation_layout()[i, j])
     params = dict(
         banner=BANNER, B=B,
         tile_layout=f"OrderBy(Row({B}, {B})).TileBy([{B}, {B}])[i, j]",
         matrix_layout=f"OrderBy(Row(cols, cols)).TileBy([cols, cols])[{B}*by + 1 + ty, {B}*bx + 1 + tx]",
-        cell=code(cell), lds=code(lds),
+        cell_row=code(cell_row), cell_lane=code(cell_lane), lds=code(lds),
     )
     text = template("nw.hip.j2").render(**params)
     return Emitted("nw_i32.hip", text, ["lego_nw_i32_launch"]), dict(B=B)
