@@ -74,11 +74,13 @@ def test_gpu_rejects_bad_sizes():
 
 
 @pytest.mark.gpu
-def test_gpu_large_matrix_reproduces_its_factors():
-    """n = 16384, the size the reference publishes: L*U gives the matrix back (fp32, diagonally dominant)."""
+@pytest.mark.parametrize("n", [5056, 8256, 16384])
+def test_gpu_large_matrix_reproduces_its_factors(n):
+    """Sizes at which the panels of the next pair of steps are solved on a second stream (79 and 129 blocks: odd
+    counts, the first just past the threshold) and n = 16384, the size the reference publishes: L*U gives the
+    matrix back (fp32, diagonally dominant)."""
     from lego_amd import ops
-    print("lud n=16384", flush=True)
-    n = 16384
+    print(f"lud n={n}", flush=True)
     a = torch.rand(n, n, device="cuda", generator=torch.Generator(device="cuda").manual_seed(61))
     a.diagonal().add_(float(n))
     w = a.clone()
