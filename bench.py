@@ -313,28 +313,21 @@ def main():
         kernels["next_needleman_wunsch_8192"] = dict(ms=ms, gcells_per_s=nn * nn / ms / 1e6,
                                                      note="255 launches, one per anti-diagonal of 64x64 tiles")
         del refm, mat
-        nl = 4096
-        a0 = torch.rand(nl, nl, generator=gen(10)).to(dev) + nl * torch.eye(nl, device=dev)
-        wk = torch.empty_like(a0)
-
-        def luf():
-            wk.copy_(a0)
-            runtime.call("lego_hip_lud_f32", p(wk), nl, stream)
-        ms = timed(luf, steps=3, warmup=1) - timed(lambda: wk.copy_(a0), steps=3, warmup=1)
-        kernels["next_lud_f32_4096"] = dict(ms=ms, tflops=(2 / 3) * nl ** 3 / ms / 1e9,
-                                            note="time of a matrix copy subtracted")
-        del a0, wk
-        # the size the reference publishes (653.5 ms for its LEGO kernel on an A100,
+        # the three sizes the reference publishes (29.7, 111.2 and 653.5 ms for its LEGO kernel on an A100,
         # benchmarks/cuda/lud/PerformanceSummary.txt:24-36)
-        nl = 16384
-        a0 = torch.rand(nl, nl, generator=gen(11)).to(dev)
-        a0.diagonal().add_(float(nl))
-        wk = torch.empty_like(a0)
-        ms = timed(luf, steps=2, warmup=1) - timed(lambda: wk.copy_(a0), steps=2, warmup=1)
-        kernels["next_lud_f32_16384"] = dict(ms=ms, tflops=(2 / 3) * nl ** 3 / ms / 1e9,
-                                             reference_ms_a100=653.5,
-                                             note="time of a matrix copy subtracted; 255 block steps of two launches")
-        del a0, wk
+        for nl, ref_ms, seed in ((4096, 29.746, 10), (8192, 111.202, 12), (16384, 653.476, 11)):
+            a0 = torch.rand(nl, nl, generator=gen(seed)).to(dev)
+            a0.diagonal().add_(float(nl))
+            wk = torch.empty_like(a0)
+
+            def luf():
+                wk.copy_(a0)
+                runtime.call("lego_hip_lud_f32", p(wk), nl, stream)
+            reps = 3 if nl < 16384 else 2
+            ms = timed(luf, steps=reps, warmup=1) - timed(lambda: wk.copy_(a0), steps=reps, warmup=1)
+            kernels[f"next_lud_f32_{nl}"] = dict(ms=ms, tflops=(2 / 3) * nl ** 3 / ms / 1e9, reference_ms_a100=ref_ms,
+                                                 note="time of a matrix copy subtracted; block steps of 64 in pairs")
+            del a0, wk
 
     # ---- CPU baseline: the oracle on a bounded panel of the headline matrix ------------------------------
     cpu = None
