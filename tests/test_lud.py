@@ -89,3 +89,37 @@ def test_gpu_large_matrix_reproduces_its_factors(n):
     lower.diagonal().fill_(1.0)
     back = lower @ torch.triu(w)
     assert ((back - a).norm() / a.norm()).item() <= 1e-5
+
+
+@pytest.mark.gpu
+def test_gpu_call_with_second_stream_replays_from_a_hip_graph():
+    """At n = 8256 the call forks to the library's second stream and joins it back with events; captured into a
+    graph (after an eager call, which creates that stream), every replay gives the bits of the eager result, with
+    eager work and synchronisation between the replays."""
+    from lego_amd import ops
+    print("lud n=8256 captured into a graph", flush=True)
+    n = 8256
+    a = torch.rand(n, n, device="cuda", generator=torch.Generator(device="cuda").manual_seed(62))
+    a.diagonal().add_(float(n))
+    w = a.clone()
+    ops.lud(w)
+    torch.cuda.synchronize()
+    want = w.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        w.copy_(a)
+        ops.lud(w)                       # warm-up on a side stream, outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.lud(w)
+    for trial in range(3):
+        w.copy_(a)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(w, want), trial
+        other = a[:512, :512] @ a[:512, :512]   # eager work between the replays
+        torch.cuda.synchronize()
+        del other
