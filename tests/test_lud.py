@@ -51,6 +51,37 @@ def test_coarsening_places_every_block_element_once():
     assert len(seen) == (R * T) ** 2
 
 
+def test_trailing_walk_covers_the_square_once():
+    """The walk of the trailing update (groups of GROUP block rows, a column of a group in parts of `run` blocks)
+    after the remap onto the XCDs: the layouts that print the kernel's index expressions, evaluated for every
+    workgroup of the padded grid, give every block of a q x q square to exactly one workgroup, and one XCD
+    (every XCDS-th workgroup id) gets a contiguous piece of the walk."""
+    import sympy as sp
+    ng, q, nsub, per, pid, wg = sp.symbols("ng q nsub per pid wg", integer=True, nonnegative=True)
+    order = sp.lambdify([ng, q, nsub, pid], lud_gen.block_order(ng, q, nsub, pid), "math")
+    remap = sp.lambdify([per, wg], lud_gen.xcd_remap(per, wg), "math")
+    G, X = lud_gen.GROUP, lud_gen.XCDS
+    for side in (1, 2, 7, 8, 9, 31, 64, 75, 124):
+        for run in (1, 2, 4, 8):
+            groups, parts = -(-side // G), G // run
+            positions = groups * side * parts
+            grid = -(-positions // X) * X
+            seen, by_xcd = set(), {}
+            for w in range(grid):
+                pos = int(remap(grid // X, w))
+                by_xcd.setdefault(w % X, []).append(pos)
+                if pos >= positions:
+                    continue
+                g, c, part = (int(v) for v in order(groups, side, parts, pos))
+                first = G * g + run * part
+                for r in range(first, min(first + run, side)):
+                    assert 0 <= c < side and (r, c) not in seen
+                    seen.add((r, c))
+            assert len(seen) == side * side, (side, run)
+            for x, got in by_xcd.items():
+                assert got == list(range(x * (grid // X), (x + 1) * (grid // X)))
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("n", [64, 128, 512, 1024])
 def test_gpu_matches_oracle(n):
