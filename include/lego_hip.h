@@ -129,6 +129,18 @@ int lego_hip_stencil_laplacian_f32(const float* in, float* out, const float* c, 
  * into `stream` with events inside the call, so the caller sees ordinary stream order. */
 int lego_hip_lud_f32(float* m, int n, void* stream);
 
+/* The launches that lego_hip_lud_f32 enqueues for an n x n matrix, in order, without touching a device: six
+ * ints per launch, {kind, stream, a, b, c, d}, stream 0 = the caller's, 1 = the library's second one.
+ *   kind 0 panels of step a (b workgroups);  1 strip: block row and column a+1 against step a (b = blocks left in
+ *   a block row);  2 the two block rows and columns at the top and left of the square of side c from block b on,
+ *   against steps a, a+1;  3 trailing update of the square of side c from block b on against d/16 steps from a on,
+ *   d%16 blocks per workgroup;  4 fork (stream 1 waits for stream 0);  5 join (stream 0 waits for stream 1);
+ *   6 factors of the a diagonal blocks written.
+ * At most `capacity` records are written; *count receives how many there are.  No counterpart in the
+ * reference (its host loop, lud_kernel_temp.cu:358-390, is three launches per step on one stream): it is
+ * there so that the order and the overlap of the launches can be checked on the host. */
+int lego_hip_lud_f32_plan(int n, int* records, int capacity, int* count);
+
 /* Needleman-Wunsch score matrix (Rodinia's needle, the reference's anti-diagonal layout
  * benchmark: benchmarks/cuda/nw_sympy.py:9-11, kernels needle_kernel_temp.cu:70-258, host
  * needle.cu:165-260).  reference and matrix are (n+1) x (n+1) int32, row-major; row 0 and

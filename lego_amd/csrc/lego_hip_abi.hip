@@ -324,6 +324,13 @@ int lego_hip_lud_f32(float* m, int n, void* stream)
   return ok_or(lego_lud_f32_launch(m, n, as_stream(stream)));
 }
 
+int lego_hip_lud_f32_plan(int n, int* records, int capacity, int* count)
+{
+  if (!count || capacity < 0 || (capacity > 0 && !records)) return kInvalid;
+  if (n <= 0 || n % LEGO_LUD_BLOCK || n > 32768) return kInvalid;
+  return ok_or(lego_lud_f32_plan(n, records, capacity, count));
+}
+
 int lego_hip_nw_i32(const int* reference, int* matrix, int n, int penalty, void* stream)
 {
   if (!usable(reference) || !usable(matrix)) return kInvalid;

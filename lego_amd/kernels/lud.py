@@ -81,4 +81,4 @@ def emit():
         xcd_layout=f"OrderBy(Col(per, {XCDS})).TileBy([per, {XCDS}])[Row(per, {XCDS}).inv(wg)]",
     )
     text = template("lud.hip.j2").render(**params)
-    return Emitted("lud_f32.hip", text, ["lego_lud_f32_launch"]), dict(B=B)
+    return Emitted("lud_f32.hip", text, ["lego_lud_f32_launch", "lego_lud_f32_plan"]), dict(B=B)

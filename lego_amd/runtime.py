@@ -40,6 +40,7 @@ SIGNATURES = {
     "lego_hip_stencil_f3d_f32": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "lego_hip_stencil_laplacian_f32": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "lego_hip_lud_f32": [_c_void_p, _c_int, _c_void_p],
+    "lego_hip_lud_f32_plan": [_c_int, ctypes.POINTER(_c_int), _c_int, ctypes.POINTER(_c_int)],
     "lego_hip_nw_i32": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "lego_hip_grouped_gemm_f16": [_PTR_ARRAY, _PTR_ARRAY, _PTR_ARRAY, _INT_ARRAY, _c_int, _c_void_p],
     "lego_hip_softmax_f16_wpr": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],

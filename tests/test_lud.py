@@ -51,6 +51,94 @@ def test_coarsening_places_every_block_element_once():
     assert len(seen) == (R * T) ** 2
 
 
+def _plan(n):
+    """The launches of lego_hip_lud_f32 for an n x n matrix, as the library's own schedule records them."""
+    import ctypes
+    from lego_amd import runtime
+    count = ctypes.c_int(0)
+    runtime.call("lego_hip_lud_f32_plan", n, None, 0, ctypes.byref(count))
+    buf = (ctypes.c_int * (6 * count.value))()
+    runtime.call("lego_hip_lud_f32_plan", n, buf, count.value, ctypes.byref(count))
+    return [tuple(buf[6 * i:6 * i + 6]) for i in range(count.value)]
+
+
+def _replay(nb, plan):
+    """Replays a recorded schedule on block indices: every launch finds its inputs final, every block gets each
+    earlier step exactly once and in order, and what runs between a fork and the next join on the two streams
+    touches disjoint blocks (write/write and read/write).  Returns how many forks there were."""
+    applied = {(i, j): [] for i in range(nb) for j in range(nb)}
+    solved = {}
+
+    def update(block, steps, writes, reads):
+        i, j = block
+        assert block not in solved and block not in writes, block
+        for st in steps:
+            assert solved.get((i, st)) == st and solved.get((st, j)) == st, (block, st)
+            applied[block].append(st)
+            reads |= {(i, st), (st, j)}
+        writes.add(block)
+
+    forks, open_main, open_side = 0, None, None
+    for kind, stream, a, b, c, d in plan:
+        writes, reads = set(), set()
+        if kind == 0:       # panels of step a, b workgroups
+            assert b == nb - 1 - a
+            assert applied[(a, a)] == list(range(a))
+            reads.add((a, a))
+            for w in range(b):
+                for block in ((a, a + 1 + w), (a + 1 + w, a)):
+                    assert applied[block] == list(range(a)) and block not in solved, block
+                    solved[block] = a
+                    writes.add(block)
+        elif kind == 1:     # block row and column a+1 against step a
+            assert b == nb - 1 - a
+            for w in range(2 * b - 1):
+                update((a + 1, a + 1 + w) if w < b else (a + 2 + w - b, a + 1), [a], writes, reads)
+        elif kind == 2:     # two block rows and columns of the square of side c from block b on
+            for w in range(4 * c - 4):
+                block = (b + w // c, b + w % c) if w < 2 * c else (b + 2 + (w - 2 * c) // 2, b + (w - 2 * c) % 2)
+                update(block, [a, a + 1], writes, reads)
+        elif kind == 3:     # the square of side c from block b on
+            depth, run = d // 16, d % 16
+            assert run in (1, 2, 4, 8) and b + c == nb
+            for i in range(c):
+                for j in range(c):
+                    update((b + i, b + j), list(range(a, a + depth)), writes, reads)
+        elif kind == 4:
+            assert open_main is None
+            forks, open_main, open_side = forks + 1, (set(), set()), (set(), set())
+            continue
+        elif kind == 5:
+            assert open_main is not None
+            (mw, mr), (sw, sr) = open_main, open_side
+            assert not (mw & sw) and not (mw & sr) and not (mr & sw)
+            open_main = open_side = None
+            continue
+        else:
+            assert kind == 6 and a == nb and open_main is None
+            continue
+        if open_main is None:
+            assert stream == 0            # the side stream is only used between a fork and a join
+        else:
+            side = open_side if stream == 1 else open_main
+            side[0].update(writes)
+            side[1].update(reads)
+    assert open_main is None and plan[-1][0] == 6
+    for (i, j), steps in applied.items():
+        assert steps == list(range(min(i, j))), (i, j)
+    for i in range(nb):
+        for j in range(nb):
+            if i != j:
+                assert solved[(i, j)] == min(i, j)
+    return forks
+
+
+@pytest.mark.parametrize("nb", list(range(1, 12)) + [63, 64, 76, 77, 78, 79, 100, 129, 256])
+def test_launch_order_updates_every_block_in_order_and_overlaps_only_disjoint_work(nb):
+    forks = _replay(nb, _plan(64 * nb))
+    assert (forks > 0) == (nb >= lud_gen.AHEAD_MIN + 5)
+
+
 def test_trailing_walk_covers_the_square_once():
     """The walk of the trailing update (groups of GROUP block rows, a column of a group in parts of `run` blocks)
     after the remap onto the XCDs: the layouts that print the kernel's index expressions, evaluated for every
