@@ -30,7 +30,7 @@ MFMA_FP8_PEAK_TFLOPS = 5000.0  # MI355X dense fp8 MFMA, published
 
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
 # what the same counters read for lego_hip_copy16 on 512 MiB (profiles/hbm_traffic_pmc.txt).
-HEADLINE_TRAFFIC_BYTES = 1074125055
+HEADLINE_TRAFFIC_BYTES = 1074079743
 
 
 def main():
