@@ -124,7 +124,7 @@ int lego_hip_stencil_laplacian_f32(const float* in, float* out, const float* c, 
  * strict lower triangle holds L (unit diagonal implied) and the upper triangle holds U, as
  * Rodinia's lud (the reference's thread-coarsening benchmark: benchmarks/cuda/lud.py:5-12,
  * kernels lud/lud_kernel_temp.cu:14-352, host loop :358-390).  n a multiple of 64, at most 32768.
- * From n = 5056 on, part of the work is enqueued on a second stream that the library creates on the
+ * From n = 4928 on, part of the work is enqueued on a second stream that the library creates on the
  * first such call on a device and keeps until the process ends; it is forked from and joined back
  * into `stream` with events inside the call, so the caller sees ordinary stream order. */
 int lego_hip_lud_f32(float* m, int n, void* stream);
