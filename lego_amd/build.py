@@ -157,8 +157,15 @@ def generate():
     return [u.write() for u in units]
 
 
-def _compile(src: Path) -> Path:
+def _compile(src: Path, incremental: bool = False) -> Path:
     obj = OBJ_DIR / (src.stem + ".o")
+    if incremental and obj.exists():
+        # the generated text is only rewritten when it changes, so modification times tell
+        # (only the hand-written ABI file includes the two headers)
+        deps = [src] + ([GENERATED / "launchers.h", ROOT / "include" / "lego_hip.h"] if src.parent == CSRC else [])
+        newest = max(p.stat().st_mtime for p in deps)
+        if obj.stat().st_mtime > newest:
+            return obj
     cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", str(ROOT / "include"), "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
@@ -166,12 +173,13 @@ def _compile(src: Path) -> Path:
     return obj
 
 
-def build(verbose=True):
-    """Generate, compile every translation unit for gfx950 and link liblego_hip.so."""
+def build(verbose=True, incremental=False):
+    """Generate, compile every translation unit for gfx950 and link liblego_hip.so.  With
+    ``incremental`` a translation unit whose object file is newer than its source is kept."""
     sources = generate() + [CSRC / "lego_hip_abi.hip"]
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
     with ThreadPoolExecutor(max_workers=8) as pool:
-        objs = list(pool.map(_compile, sources))
+        objs = list(pool.map(lambda s: _compile(s, incremental), sources))
     cmd = [hipcc_path(), f"--offload-arch=gfx950", "-shared", "-fPIC", *[str(o) for o in objs], "-o", str(LIB_PATH)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
@@ -184,10 +192,11 @@ def build(verbose=True):
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--emit", action="store_true", help="generate sources only")
+    ap.add_argument("--incremental", action="store_true", help="recompile only the sources that changed")
     ns = ap.parse_args()
     if ns.emit:
         for p in generate():
             print(p)
     else:
-        build()
+        build(incremental=ns.incremental)
     sys.exit(0)
