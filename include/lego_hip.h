@@ -69,6 +69,18 @@ int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, con
                                const float* rstd, void* dx, void* dw, void* db, void* workspace,
                                unsigned long long workspace_bytes, int M, int N, void* stream);
 
+/* lego_hip_layernorm_bwd_f16 without the workspace argument, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  The fp32 partial rows live in a 32 MiB array inside the library's
+ * code object, one copy per device, held until the process ends; every fp16 shape that
+ * lego_hip_layernorm_bwd_f16 takes needs at most that much (a shape that needed more would return
+ * hipErrorInvalidValue).  The device that owns `stream` must be the current device of the calling
+ * thread.  Calls on one device share the array: two calls that overlap in time on one device (on
+ * different streams) race on it and must be ordered by the caller.  The call itself allocates and
+ * frees nothing and does not synchronise. */
+int lego_hip_layernorm_bwd_f16_noalloc(const void* dy, const void* x, const void* w, const float* mean,
+                                       const float* rstd, void* dx, void* dw, void* db, int M, int N, void* stream);
+
 /* The same for fp32 tensors (the reference's kernels take the tensors' own type, layernorm.py:372-405);
  * every shape takes the two passes; the workspace has its own size. */
 int lego_hip_layernorm_bwd_f32_workspace_bytes(int M, int N, unsigned long long* bytes);

@@ -8,6 +8,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "lego_hip.h"
 #include "generated/launchers.h"
 
@@ -37,6 +39,35 @@ __global__ void __launch_bounds__(256) lego_copy16_stream_kernel(const u32x4* __
   for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(in + base + u * 256);
 #pragma unroll
   for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(v[u], out + base + u * 256);
+}
+
+// Scratch of lego_hip_layernorm_bwd_f16_noalloc: the fp32 dw/db partial rows that the other
+// LayerNorm backward entry points take from the caller.  One copy per device, held until the process
+// ends.  In host code the array's name is only a handle for hipGetSymbolAddress; kernels and launchers
+// receive the device address kept in scratch_ptr[device].
+constexpr unsigned long long kScratchBytes = 32ull << 20;
+static __device__ __align__(256) float scratch[kScratchBytes / sizeof(float)];
+constexpr int kMaxDevices = 64;
+float* scratch_ptr[kMaxDevices];
+std::mutex scratch_mutex;
+
+// Device address of the current device's scratch array (looked up on the first call per device).
+hipError_t scratch_address(float** out)
+{
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> hold(scratch_mutex);
+  if (scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return err;
+    if (p == nullptr) return hipErrorInvalidSymbol;
+    scratch_ptr[dev] = static_cast<float*>(p);
+  }
+  *out = scratch_ptr[dev];
+  return hipSuccess;
 }
 
 }  // namespace
@@ -185,6 +216,22 @@ int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, con
   if (mean == nullptr || rstd == nullptr || workspace_bytes < need) return kInvalid;
   return ok_or(lego_layernorm_bwd_f16_launch(dy, x, w, mean, rstd, dx, dw, db, static_cast<float*>(workspace), M, N,
                                              as_stream(stream)));
+}
+
+int lego_hip_layernorm_bwd_f16_noalloc(const void* dy, const void* x, const void* w, const float* mean,
+                                       const float* rstd, void* dx, void* dw, void* db, int M, int N, void* stream)
+{
+  unsigned long long need = 0;
+  if (lego_hip_layernorm_bwd_workspace_bytes(M, N, &need) != 0) return kInvalid;
+  if (need > kScratchBytes) return kInvalid;     // partial rows beyond the built-in scratch
+  if (!usable(dy) || !usable(x) || !usable(w) || !usable(dx) || !usable(dw) || !usable(db)) return kInvalid;
+  if (mean == nullptr || rstd == nullptr) return kInvalid;
+  float* partials = nullptr;
+  const hipError_t err = scratch_address(&partials);
+  if (err != hipSuccess) return ok_or(err);
+  // every partial row that the reduction reads is written by the first stage of the same call, so
+  // what an earlier call left in the array needs no clearing
+  return ok_or(lego_layernorm_bwd_f16_launch(dy, x, w, mean, rstd, dx, dw, db, partials, M, N, as_stream(stream)));
 }
 
 int lego_hip_layernorm_bwd_f32_workspace_bytes(int M, int N, unsigned long long* bytes)

@@ -48,6 +48,7 @@ SIGNATURES = {
                                        _c_int, _c_int, _c_float, _c_int, _c_void_p],
     "lego_hip_layernorm_bwd_workspace_bytes": [_c_int, _c_int, ctypes.POINTER(ctypes.c_ulonglong)],
     "lego_hip_layernorm_bwd_f16": [_c_void_p] * 9 + [ctypes.c_ulonglong, _c_int, _c_int, _c_void_p],
+    "lego_hip_layernorm_bwd_f16_noalloc": [_c_void_p] * 8 + [_c_int, _c_int, _c_void_p],
     "lego_hip_layernorm_bwd_f32_workspace_bytes": [_c_int, _c_int, ctypes.POINTER(ctypes.c_ulonglong)],
     "lego_hip_layernorm_bwd_f32": [_c_void_p] * 9 + [ctypes.c_ulonglong, _c_int, _c_int, _c_void_p],
     "lego_hip_layernorm_bwd_bf16_workspace_bytes": [_c_int, _c_int, ctypes.POINTER(ctypes.c_ulonglong)],
