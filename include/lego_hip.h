@@ -170,6 +170,17 @@ int lego_hip_nw_i32(const int* reference, int* matrix, int n, int penalty, void*
 int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* const* c,
                               const int* sizes3, int groups, void* stream);
 
+/* What lego_hip_grouped_gemm_f16 launches for these sizes, without touching a device: plan3[0] = tile
+ * size (256: 256 x 256 tiles, or 128: 128 x 128 tiles), plan3[1] = number of 256 x 256 tiles of all
+ * problems, plan3[2] = how many of them, the last ones of the launch order, are computed as two
+ * 128 x 256 halves by two workgroups.  No counterpart in the reference (its kernel walks whole tiles
+ * only, grouped_gemm.py:61-116); it is there so that the launch can be checked on the host. */
+int lego_hip_grouped_gemm_f16_plan(const int* sizes3, int groups, int* plan3);
+/* Tuning entry point: lego_hip_grouped_gemm_f16 with the launch chosen by the caller: split_tiles >= 0
+ * = 256 x 256 tiles, the last split_tiles of them as halves; split_tiles < 0 = 128 x 128 tiles. */
+int lego_hip_grouped_gemm_f16_split(const void* const* a, const void* const* b, void* const* c,
+                                    const int* sizes3, int groups, int split_tiles, void* stream);
+
 /* Tuning entry points: as above, with the launch shape chosen by the caller
  * (waves_per_row in {1, 2, 4, 16}; N a multiple of 8 and at most 8192 * waves_per_row, 16384 for 4).  Used by the benchmark to compare variants. */
 int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per_row, void* stream);

@@ -76,7 +76,8 @@ def generate():
         for ta in (False, True):
             for tb in (False, True):
                 g, m_ = gemm.emit(**dict(GEMM, bk=GEMM_BK[dtype]), trans_a=ta, trans_b=tb, dtype=dtype,
-                                  with_grouped=dtype == "f16" and not (ta or tb))
+                                  with_grouped=dtype == "f16" and not (ta or tb),
+                                  with_split=dtype == "f16" and not (ta or tb))
                 units.append(g)
                 if dtype == "f16":
                     mg = m_
@@ -141,6 +142,8 @@ def generate():
           "const int*, int, hipStream_t);",
           f"hipError_t lego_grouped_gemm_f16_t{GEMM_SMALL_TILE}x{GEMM_SMALL_TILE}_launch(const void* const*, "
           "const void* const*, void* const*, const int*, int, hipStream_t);",
+          "hipError_t lego_grouped_gemm_f16_split_launch(const void* const*, const void* const*, void* const*, "
+          "const int*, int, int, hipStream_t);",
           f"#define LEGO_GEMM_BM {mg['BM']}", f"#define LEGO_GEMM_BN {mg['BN']}", f"#define LEGO_GEMM_BK {mg['BK']}",
           f"#define LEGO_GEMM_BK_8BIT {GEMM_BK['e5m2']}",
           f"#define LEGO_GROUPED_MAX_GROUPS {mg['MAX_GROUPS']}", ""]

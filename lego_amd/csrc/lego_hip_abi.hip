@@ -386,21 +386,21 @@ int lego_hip_nw_i32(const int* reference, int* matrix, int n, int penalty, void*
 }
 
 namespace {
-// Time of a launch of the grouped kernel, in k-tiles of one workgroup: list scheduling of its
-// tiles, in launch order, on `slots` workgroups that run at once (a tile goes to the slot that
-// frees up first).  tiles[g] tiles of depth[g] k-tiles each.  The slot loads are kept as a
-// sorted list of (load, how many slots) levels, so a group of equal tiles costs a few steps.
-static double grouped_makespan(const long* tiles, const long* depth, int groups, long slots)
+// Time of a grouped launch: list scheduling of its workgroups, in launch order, on `slots` workgroups
+// that run at once (a workgroup goes to the slot that frees up first).  The launch is a sequence of
+// batches of count[i] workgroups that take cost[i] each.  The slot loads are kept as a sorted list of
+// (load, how many slots) levels, so a batch of equal workgroups costs a few steps.
+double grouped_makespan(const long* count, const double* cost, int batches, long slots)
 {
   struct Level { double load; long count; };
-  Level lv[4 * LEGO_GROUPED_MAX_GROUPS + 4];
+  Level lv[8 * LEGO_GROUPED_MAX_GROUPS + 8];
   int n = 1;
   lv[0] = {0.0, slots};
-  for (int g = 0; g < groups; ++g) {
-    long left = tiles[g];
-    const double d = static_cast<double>(depth[g]);
+  for (int g = 0; g < batches; ++g) {
+    long left = count[g];
+    const double d = cost[g];
     while (left > 0) {
-      // the least loaded level takes tiles, one per slot; its slots move up by d
+      // the least loaded level takes workgroups, one per slot; its slots move up by d
       const long take = left < lv[0].count ? left : lv[0].count;
       const double moved = lv[0].load + d;
       lv[0].count -= take;
@@ -426,10 +426,76 @@ static double grouped_makespan(const long* tiles, const long* depth, int groups,
   }
   return lv[n - 1].load;
 }
-}  // namespace
 
-int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* const* c,
-                              const int* sizes3, int groups, void* stream)
+// What a grouped call launches: the kernel on 256 x 256 tiles with the last `split` tiles of its launch
+// order as two 128 x 256 halves each (kind 0), or the kernel on 128 x 128 tiles (kind 1).
+struct GroupedPlan {
+  int kind, tiles, split;
+  int order[LEGO_GROUPED_MAX_GROUPS];       // problems in launch order: decreasing depth, stable
+};
+
+// Costs in units of one k-tile step of a 256 x 256 tile that has its CU to itself (about 1.8 us for
+// fp16), measured on MI355X: a tile pays a start-up and an epilogue on top of its steps (31.4 us for
+// 16 steps); a 128 x 256 half-tile takes 19.2 us for 16 steps; a 128 x 128 tile sharing its CU with
+// another one takes 0.66 of a whole tile of the same depth.
+constexpr double kTileOverhead = 1.6, kHalfStep = 0.58, kHalfOverhead = 1.5, kSmallCost = 0.66;
+
+GroupedPlan grouped_plan(const int* sizes3, int groups)
+{
+  GroupedPlan plan;
+  for (int g = 0; g < groups; ++g) plan.order[g] = g;
+  for (int i = 1; i < groups; ++i) {
+    const int o = plan.order[i];
+    int j = i;
+    while (j > 0 && sizes3[3 * plan.order[j - 1] + 2] < sizes3[3 * o + 2]) { plan.order[j] = plan.order[j - 1]; --j; }
+    plan.order[j] = o;
+  }
+  long big[LEGO_GROUPED_MAX_GROUPS], small[LEGO_GROUPED_MAX_GROUPS];
+  double depth[LEGO_GROUPED_MAX_GROUPS], small_cost[LEGO_GROUPED_MAX_GROUPS];
+  long total = 0;
+  for (int s = 0; s < groups; ++s) {
+    const int g = plan.order[s];
+    const int m = sizes3[3 * g], n = sizes3[3 * g + 1];
+    big[s] = static_cast<long>((m + 255) / 256) * ((n + 255) / 256);
+    small[s] = static_cast<long>((m + 127) / 128) * ((n + 127) / 128);
+    depth[s] = sizes3[3 * g + 2] / LEGO_GEMM_BK;
+    small_cost[s] = kSmallCost * (depth[s] + kTileOverhead);
+    total += big[s];
+  }
+  const long cus = 256;                 // MI355X
+  // 256 x 256 tiles, the last `split` of them as halves: the best split among multiples of 16 tiles
+  // up to two rounds of the CUs
+  double best = 0.0;
+  long best_split = 0;
+  const long max_split = total < 2 * cus ? total : 2 * cus;
+  for (long split = 0; split <= max_split; split += 16) {
+    long count[2 * LEGO_GROUPED_MAX_GROUPS];
+    double cost[2 * LEGO_GROUPED_MAX_GROUPS];
+    int nb = 0;
+    long whole_left = total - split;
+    for (int s = 0; s < groups; ++s) {
+      const long w = big[s] < whole_left ? big[s] : whole_left;
+      whole_left -= w;
+      if (w > 0) { count[nb] = w; cost[nb++] = depth[s] + kTileOverhead; }
+    }
+    whole_left = total - split;
+    for (int s = 0; s < groups; ++s) {
+      const long w = big[s] < whole_left ? big[s] : whole_left;
+      whole_left -= w;
+      if (big[s] > w) { count[nb] = 2 * (big[s] - w); cost[nb++] = kHalfStep * depth[s] + kHalfOverhead; }
+    }
+    const double t = grouped_makespan(count, cost, nb, cus);
+    // equal estimates: the larger split (more, shorter workgroups in the last round measured faster)
+    if (split == 0 || t <= best) { best = t; best_split = split; }
+  }
+  const double t_small = grouped_makespan(small, small_cost, groups, 2 * cus);
+  plan.kind = t_small < best ? 1 : 0;
+  plan.tiles = static_cast<int>(total);
+  plan.split = plan.kind == 0 ? static_cast<int>(best_split) : 0;
+  return plan;
+}
+
+int grouped_check(const void* const* a, const void* const* b, void* const* c, const int* sizes3, int groups)
 {
   if (a == nullptr || b == nullptr || c == nullptr || sizes3 == nullptr) return kInvalid;
   if (groups <= 0 || groups > LEGO_GROUPED_MAX_GROUPS) return kInvalid;
@@ -438,43 +504,45 @@ int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* 
     if (!usable(a[g]) || !usable(b[g]) || !usable(c[g])) return kInvalid;
     if (m <= 0 || n <= 0 || k <= 0 || m % 8 || n % 8 || k % LEGO_GEMM_BK) return kInvalid;
   }
-  // One launch, on 256 x 256 tiles (one workgroup per CU) or on 128 x 128 tiles (four times as many
-  // workgroups of a quarter of the work, two per CU), whichever the estimate below finishes first:
-  // small tiles win when the big ones leave most CUs idle or the last round mostly empty.  Problems
-  // are launched in order of decreasing depth, so the longest tiles start first.  (Splitting the
-  // problems over both kernels was measured and never beat the better of the two single launches.)
-  int order[LEGO_GROUPED_MAX_GROUPS];
-  for (int g = 0; g < groups; ++g) order[g] = g;
-  for (int i = 1; i < groups; ++i) {
-    const int o = order[i];
-    int j = i;
-    while (j > 0 && sizes3[3 * order[j - 1] + 2] < sizes3[3 * o + 2]) { order[j] = order[j - 1]; --j; }
-    order[j] = o;
-  }
-  long big[LEGO_GROUPED_MAX_GROUPS], small[LEGO_GROUPED_MAX_GROUPS], depth[LEGO_GROUPED_MAX_GROUPS];
-  const void* pa[LEGO_GROUPED_MAX_GROUPS];
-  const void* pb[LEGO_GROUPED_MAX_GROUPS];
-  void* pc[LEGO_GROUPED_MAX_GROUPS];
-  int sz[3 * LEGO_GROUPED_MAX_GROUPS];
-  for (int s = 0; s < groups; ++s) {
-    const int g = order[s];
-    const int m = sizes3[3 * g], n = sizes3[3 * g + 1];
-    big[s] = static_cast<long>((m + 255) / 256) * ((n + 255) / 256);
-    small[s] = static_cast<long>((m + 127) / 128) * ((n + 127) / 128);
-    depth[s] = sizes3[3 * g + 2] / LEGO_GEMM_BK;
-    pa[s] = a[g];
-    pb[s] = b[g];
-    pc[s] = c[g];
-    for (int e = 0; e < 3; ++e) sz[3 * s + e] = sizes3[3 * g + e];
-  }
-  const long cus = 256;                 // MI355X
-  // a 128 x 128 tile sharing its CU with another one, against a 256 x 256 tile of the same depth
-  // that has the CU to itself (measured: 45 us against 68 us for 40 k-tiles)
-  const double small_cost = 0.66;
-  const bool use_small = small_cost * grouped_makespan(small, depth, groups, 2 * cus) <
-                         grouped_makespan(big, depth, groups, cus);
-  return ok_or((use_small ? lego_grouped_gemm_f16_t128x128_launch : lego_grouped_gemm_f16_launch)(
-      pa, pb, pc, sz, groups, as_stream(stream)));
+  return 0;
+}
+}  // namespace
+
+int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* const* c,
+                              const int* sizes3, int groups, void* stream)
+{
+  if (grouped_check(a, b, c, sizes3, groups) != 0) return kInvalid;
+  // One launch: on 256 x 256 tiles (one workgroup per CU), the last tiles of the launch order split
+  // into halves when whole tiles would leave the last round mostly empty, or on 128 x 128 tiles (four
+  // times as many workgroups of a quarter of the work, two per CU) when the big ones leave most CUs
+  // idle; whichever the estimate finishes first.  Problems are launched in order of decreasing
+  // depth, so the longest tiles start first.  (Splitting the problems over both tile sizes in two
+  // launches was measured and never beat the better single launch.)
+  const GroupedPlan plan = grouped_plan(sizes3, groups);
+  if (plan.kind == 1) return ok_or(lego_grouped_gemm_f16_t128x128_launch(a, b, c, sizes3, groups, as_stream(stream)));
+  if (plan.split == 0) return ok_or(lego_grouped_gemm_f16_launch(a, b, c, sizes3, groups, as_stream(stream)));
+  return ok_or(lego_grouped_gemm_f16_split_launch(a, b, c, sizes3, groups, plan.split, as_stream(stream)));
+}
+
+int lego_hip_grouped_gemm_f16_plan(const int* sizes3, int groups, int* plan3)
+{
+  if (sizes3 == nullptr || plan3 == nullptr || groups <= 0 || groups > LEGO_GROUPED_MAX_GROUPS) return kInvalid;
+  for (int g = 0; g < groups; ++g)
+    if (sizes3[3 * g] <= 0 || sizes3[3 * g + 1] <= 0 || sizes3[3 * g + 2] <= 0) return kInvalid;
+  const GroupedPlan plan = grouped_plan(sizes3, groups);
+  plan3[0] = plan.kind == 1 ? 128 : 256;
+  plan3[1] = plan.tiles;
+  plan3[2] = plan.split;
+  return 0;
+}
+
+int lego_hip_grouped_gemm_f16_split(const void* const* a, const void* const* b, void* const* c,
+                                    const int* sizes3, int groups, int split_tiles, void* stream)
+{
+  if (grouped_check(a, b, c, sizes3, groups) != 0) return kInvalid;
+  if (split_tiles < 0)
+    return ok_or(lego_grouped_gemm_f16_t128x128_launch(a, b, c, sizes3, groups, as_stream(stream)));
+  return ok_or(lego_grouped_gemm_f16_split_launch(a, b, c, sizes3, groups, split_tiles, as_stream(stream)));
 }
 
 int lego_hip_copy16(const void* in, void* out, unsigned long long bytes, void* stream)

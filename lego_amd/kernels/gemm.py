@@ -104,8 +104,8 @@ def xcd_remap(per, wg, xcds=XCDS):
     return OrderBy(Col(per, xcds)).TileBy([per, xcds])[j, x]
 
 
-def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, trans_b=False, with_grouped=True,
-         dtype="f16"):
+def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped, dtype):
+    """Everything the templates need for one tile shape."""
     # element type, bytes per element, k-depth of one MFMA, result type; the 8-bit types are the
     # OCP formats of v_mfma_f32_32x32x64_f8f6f4 (format code 0 = e4m3, 1 = e5m2)
     elt, esize, mfma_k, out_elt = {"f16": ("_Float16", 2, 16, "_Float16"), "bf16": ("__bf16", 2, 16, "__bf16"),
@@ -286,7 +286,44 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
         xcd_pid=code(tidy(xcd_remap(per_xcd, wg), {wg: (0, per_xcd * XCDS)})),
         pid_m=code(pm_e), pid_n=code(pn_e),
     )
+    return params
+
+
+def split_order(split, wg):
+    """``(tile, half)`` of workgroup ``wg`` among the ``2*split`` workgroups that share ``split``
+    tiles between two halves each: ``Row(split, 2).inv(wg)``."""
+    return OrderBy(Row(split, 2)).TileBy([split, 2]).inv(wg)
+
+
+def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, trans_b=False, with_grouped=True,
+         dtype="f16", with_split=False):
+    """One translation unit: the GEMM kernel of one operand layout and element type on ``bm x bn``
+    tiles, with ``with_grouped`` the grouped kernel on the same tiles, and with ``with_split`` a
+    second grouped kernel that gives the last tiles of its launch to two workgroups each, as
+    halves of ``bm/2 x bn`` (the tail of a launch whose last round of whole tiles would leave most
+    CUs idle)."""
+    params = _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped, dtype)
+    ns = f"t{bm}x{bn}"
+    tiles = [dict(ns=ns, text=template("gemm_tile.hip.j2").render(**params))]
+    params.update(main_ns=ns, with_split=with_split)
+    if with_split:
+        assert with_grouped
+        half = _tile_params(bm // 2, bn, bk, waves, max_group_m, trans_a, trans_b, True, dtype)
+        hns = f"t{bm // 2}x{bn}"
+        tiles.append(dict(ns=hns, text=template("gemm_tile.hip.j2").render(**half)))
+        split, swg, ti, hf = size("split"), idx("swg"), idx("pid_m"), idx("half")
+        tile_e, half_e = (tidy(e, {swg: (0, 2 * split)}) for e in split_order(split, swg))
+        params.update(half_ns=hns, HBM=bm // 2,
+                      split_layout="OrderBy(Row(split, 2)).TileBy([split, 2]).inv(wg - whole)",
+                      split_tile=code(tile_e), split_half=code(half_e),
+                      # rows of halves in place of rows of tiles: one more level under the tile row
+                      half_pid_m=code(tidy(OrderBy(Row(size("num_pid_m"), 2)).TileBy([size("num_pid_m"), 2])[ti, hf],
+                                           {ti: (0, size("num_pid_m")), hf: (0, 2)})))
+    params["tiles"] = tiles
     text = template("gemm.hip.j2").render(**params)
+    variant, tag = params["variant"], params["tag"]
     meta = dict(BM=bm, BN=bn, BK=bk, MAX_GROUPS=MAX_GROUPS)
     launchers = [f"lego_gemm_{dtype}_{variant}{tag}_launch"] + ([f"lego_grouped_gemm_f16{tag}_launch"] if with_grouped else [])
+    if with_split:
+        launchers.append(f"lego_grouped_gemm_f16{tag}_split_launch")
     return Emitted(f"gemm_{dtype}_{variant}{tag}.hip", text, launchers), meta

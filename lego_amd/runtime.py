@@ -43,6 +43,8 @@ SIGNATURES = {
     "lego_hip_lud_f32_plan": [_c_int, ctypes.POINTER(_c_int), _c_int, ctypes.POINTER(_c_int)],
     "lego_hip_nw_i32": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "lego_hip_grouped_gemm_f16": [_PTR_ARRAY, _PTR_ARRAY, _PTR_ARRAY, _INT_ARRAY, _c_int, _c_void_p],
+    "lego_hip_grouped_gemm_f16_plan": [_INT_ARRAY, _c_int, _INT_ARRAY],
+    "lego_hip_grouped_gemm_f16_split": [_PTR_ARRAY, _PTR_ARRAY, _PTR_ARRAY, _INT_ARRAY, _c_int, _c_int, _c_void_p],
     "lego_hip_softmax_f16_wpr": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "lego_hip_layernorm_fwd_f16_wpr": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                        _c_int, _c_int, _c_float, _c_int, _c_void_p],

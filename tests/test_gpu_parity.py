@@ -521,6 +521,90 @@ def test_grouped_gemm_many_tiles_unsorted_depths(ops):
         assert _rel_err(c.cpu(), w) <= 1e-2
 
 
+def _grouped_call(entry, A, B, *extra):
+    """Call a grouped entry point through the C ABI on device tensors; returns the results."""
+    import ctypes
+    from lego_amd import runtime
+    C = [torch.empty(a.shape[0], b.shape[1], dtype=torch.half, device="cuda") for a, b in zip(A, B)]
+    n = len(A)
+    arr = ctypes.c_void_p * n
+    sz = (ctypes.c_int * (3 * n))(*[v for a, b in zip(A, B) for v in (a.shape[0], b.shape[1], a.shape[1])])
+    runtime.call(entry, arr(*[t.data_ptr() for t in A]), arr(*[t.data_ptr() for t in B]),
+                 arr(*[t.data_ptr() for t in C]), sz, n, *extra,
+                 ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    return C
+
+
+def test_grouped_gemm_headline_problem_set_at_full_depth(ops):
+    """Config 5 as the benchmark builds it (seed 5: 8 problems from {1024, 2048, 4096}^3), whole: the
+    launch splits its last tiles into halves.  Row panels of every problem against the CPU oracle
+    (the first rows, rows 96..159 that straddle the two halves of a tile, the last rows), and the
+    whole result against an fp32 product on the device."""
+    print("grouped gemm config 5 at full depth", flush=True)
+    g = _gen(5)
+    idx = torch.randint(0, 3, (8, 3), generator=g)
+    dims = [[(1024, 2048, 4096)[int(v)] for v in row] for row in idx]
+    A = [(torch.randn(m, k, generator=g) / math.sqrt(k)).half() for m, n, k in dims]
+    B = [(torch.randn(k, n, generator=g) / math.sqrt(k)).half() for m, n, k in dims]
+    got = ops.lego_group_gemm_fn([a.cuda() for a in A], [b.cuda() for b in B])
+    for (m, n, k), a, b, c in zip(dims, A, B, got):
+        assert c.shape == (m, n)
+        for r0 in (0, 96, m - 64):
+            want = ok.gemm(a[r0:r0 + 64], b)
+            assert _rel_err(c[r0:r0 + 64].cpu(), want) <= 1e-2, (m, n, k, r0)
+            assert (c[r0:r0 + 64].cpu().float() - want.float()).abs().max().item() <= 1e-2
+        ref = a.cuda().float() @ b.cuda().float()
+        assert ((c.float() - ref).norm() / ref.norm()).item() <= 1e-2
+
+
+@pytest.mark.parametrize("split", [0, 1, 7, 24, -1])
+def test_grouped_gemm_split_tail_on_ragged_shapes(ops, split):
+    """The launch with its last `split` tiles as two halves each, forced through the tuning entry
+    point, on problems whose tiles are ragged: a last tile row of 8 rows (its lower half is empty), one
+    of 136 rows (a lower half of 8 rows), ragged columns.  24 = every tile split; -1 = 128 x 128 tiles."""
+    print(f"grouped gemm split tail {split}", flush=True)
+    g = _gen(31)
+    shapes = [(1000, 776, 192), (520, 264, 128), (136, 512, 64)]       # 16 + 6 + 2 tiles of 256 x 256
+    A = [(torch.randn(m, k, generator=g) / math.sqrt(k)).half() for m, n, k in shapes]
+    B = [(torch.randn(k, n, generator=g) / math.sqrt(k)).half() for m, n, k in shapes]
+    want = ok.grouped_gemm(A, B)
+    got = _grouped_call("lego_hip_grouped_gemm_f16_split", [a.cuda() for a in A], [b.cuda() for b in B], split)
+    for c, w in zip(got, want):
+        assert _rel_err(c.cpu(), w) <= 1e-2
+        assert (c.cpu().float() - w.float()).abs().max().item() <= 1e-2
+
+
+def test_grouped_gemm_split_matches_whole_tiles_bit_for_bit(ops):
+    """A half-tile accumulates the same k-steps in the same order as the whole tile: same bits."""
+    print("grouped gemm split vs whole", flush=True)
+    g = _gen(32)
+    shapes = [(2048, 1024, 512), (1024, 2048, 256), (512, 512, 128)]
+    A = [(torch.randn(m, k, generator=g) / math.sqrt(k)).half().cuda() for m, n, k in shapes]
+    B = [(torch.randn(k, n, generator=g) / math.sqrt(k)).half().cuda() for m, n, k in shapes]
+    whole = _grouped_call("lego_hip_grouped_gemm_f16_split", A, B, 0)
+    for split in (5, 68):
+        for c, w in zip(_grouped_call("lego_hip_grouped_gemm_f16_split", A, B, split), whole):
+            assert torch.equal(c, w)
+
+
+def test_gemm_headline_shape_8192_cubed(ops):
+    """Config 4 at full size: 1024 tiles, 128 k-steps each, operands 128 MiB apart as two consecutive
+    allocations are.  Two 256-row panels (the first tile row and one in the middle of the launch order's
+    last group) against the CPU oracle."""
+    print("gemm 8192 cubed", flush=True)
+    n = 8192
+    g = _gen(4)
+    a = (torch.randn(n, n, generator=g) / math.sqrt(n)).half()
+    b = (torch.randn(n, n, generator=g) / math.sqrt(n)).half()
+    c = ops.matmul(a.cuda(), b.cuda())
+    for r0 in (0, 7424):
+        want = ok.gemm(a[r0:r0 + 256], b)
+        got = c[r0:r0 + 256].cpu()
+        assert _rel_err(got, want) <= 1e-2
+        assert (got.float() - want.float()).abs().max().item() <= 1e-2
+
+
 def test_kernels_run_on_the_callers_stream(ops):
     """The wrappers enqueue on torch's current stream: work issued on a side stream is ordered after that
     stream's earlier work (the input is produced there) and is complete once the stream is."""

@@ -1,0 +1,83 @@
+"""The launch that lego_hip_grouped_gemm_f16 makes, replayed on the host: the plan the entry point
+reports, the workgroup -> (problem, tile, half) map of the kernels (the LEGO layouts the generator
+prints into them, evaluated with integers), and that the workgroups' blocks of C tile every problem
+exactly once."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from lego_amd import runtime
+from lego_amd.kernels import gemm
+from lego_amd.lego import OrderBy, Row
+
+C5 = [(4096, 1024, 2048), (1024, 4096, 2048), (2048, 4096, 1024), (2048, 2048, 1024), (4096, 4096, 1024),
+      (1024, 1024, 1024), (4096, 2048, 1024), (1024, 1024, 1024)]
+
+
+def _plan(sizes):
+    sz = (ctypes.c_int * (3 * len(sizes)))(*[v for s in sizes for v in s])
+    out = (ctypes.c_int * 3)()
+    runtime.call("lego_hip_grouped_gemm_f16_plan", sz, len(sizes), out)
+    return list(out)
+
+
+def _group_height(num_pid_m, max_gm=8):
+    gm = max_gm
+    while num_pid_m % gm:
+        gm -= 1
+    return gm
+
+
+def _coverage(sizes, split):
+    """Blocks of 128 x 256 of every problem's C, counted over all workgroups of the split launch."""
+    order = sorted(range(len(sizes)), key=lambda g: -sizes[g][2])        # decreasing depth, stable
+    tiles = [(-(-sizes[g][0] // 256), -(-sizes[g][1] // 256)) for g in order]
+    ends = np.cumsum([tm * tn for tm, tn in tiles])
+    total = int(ends[-1])
+    whole = total - split
+    seen = [np.zeros((2 * tm, tn), dtype=int) for tm, tn in tiles]
+    for wg in range(total + split):
+        if wg < whole:
+            tile, half = wg, None
+        else:
+            t, half = gemm.split_order(split, wg - whole)               # Row(split, 2).inv(wg - whole)
+            tile = whole + int(t)
+        s = int(np.searchsorted(ends, tile, side="right"))
+        pid = tile - (int(ends[s - 1]) if s else 0)
+        npm, npn = tiles[s]
+        pid_m, pid_n = (int(v) for v in gemm.launch_order(npm, npn, _group_height(npm), pid))
+        assert 0 <= pid_m < npm and 0 <= pid_n < npn
+        if half is None:
+            seen[s][2 * pid_m:2 * pid_m + 2, pid_n] += 1
+        else:
+            half_m = int(OrderBy(Row(npm, 2)).TileBy([npm, 2])[pid_m, int(half)])
+            seen[s][half_m, pid_n] += 1
+    return seen, total
+
+
+@pytest.mark.parametrize("sizes", [C5, [(256, 256, 64)], [(1000, 776, 192), (520, 264, 128), (136, 512, 64)],
+                                   [(2048, 2048, 512)] * 5, [(4096, 4096, 4096), (512, 512, 64)]])
+def test_every_block_of_c_is_computed_once(sizes):
+    kind, total, split = _plan(sizes)
+    assert total == sum(-(-m // 256) * -(-n // 256) for m, n, _ in sizes)
+    assert 0 <= split <= total
+    for s in sorted({0, 1, split, total // 2, total}):
+        seen, _ = _coverage(sizes, s)
+        for blocks in seen:
+            assert (blocks == 1).all()
+
+
+def test_plan_splits_the_tail_of_the_headline_problem_set():
+    kind, total, split = _plan(C5)
+    # 128 tiles of depth 32 and 608 of depth 16 on 256 CUs: three rounds and 96 tiles over; the
+    # plan gives that tail (or more) to halves
+    assert (kind, total) == (256, 736) and 96 <= split <= 224 and split % 16 == 0
+
+
+def test_plan_keeps_whole_rounds_whole_and_small_sets_on_small_tiles():
+    assert _plan([(4096, 4096, 1024)]) == [256, 256, 0]            # exactly one round of whole tiles
+    assert _plan([(8192, 8192, 2048)])[2] == 0                     # four rounds
+    assert _plan([(1024, 512, 256), (512, 512, 512)])[0] == 128    # a handful of tiles: 128 x 128 tiles
+    with pytest.raises(runtime.LegoHipError):
+        _plan([(0, 256, 64)])
