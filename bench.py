@@ -8,8 +8,11 @@ Prints ONE JSON line.  A "step" is one launch of the headline workload, the fp16
 the headline metric is quoted on); ``value`` is its effective HBM bandwidth with the input
 already resident in device memory.  The other four configurations are timed in the same
 run with the same K and W and reported under ``kernels`` with their own roofline
-fractions.  ``cpu_baseline`` times the CPU oracle (index arrays through the two layouts +
-gather/scatter) on a bounded panel of the same matrix, on this host's cores.
+fractions.  ``cpu_baseline`` times the reference's CPU path for the headline workload -- the source and
+destination offsets as LEGO's Python/Triton printer emits them, evaluated with ``torch.arange`` for
+``tl.arange``, then one gather/scatter -- on a bounded panel of the same matrix, on this host's
+cores; the other configurations carry their own ``cpu_baseline`` (PyTorch CPU operators, as the
+reference's CPU path has them) under ``kernels``.
 
 Timing uses HIP events recorded on the stream the kernels are launched on (torch's
 current stream).  Working sets that fit the 256 MB Infinity Cache are timed twice: "hot"
@@ -28,16 +31,32 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
 MFMA_FP8_PEAK_TFLOPS = 5000.0  # MI355X dense fp8 MFMA, published
 
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
-# what the same counters read for lego_hip_copy16 on 512 MiB (profiles/hbm_traffic_pmc.txt).
-HEADLINE_TRAFFIC_BYTES = 1074079743
+SETTLE_MS = 40.0               # untimed device time before every timed region, see timed()
+
+HEADLINE_KERNEL = "lego_transpose_f16_64x256_w128x8"
+TRAFFIC_PROFILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic_pmc.txt")
+
+
+def headline_traffic_bytes():
+    """HBM bytes per launch of the headline kernel, read from the committed counter summary (rocprofv3
+    --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters read for a plain copy of known
+    size): the "scaled bytes" column of the kernel's row.  None when the summary has no such row."""
+    try:
+        with open(TRAFFIC_PROFILE) as fh:
+            for line in fh:
+                if line.startswith(HEADLINE_KERNEL + " "):
+                    numbers = [int(tok) for tok in line.split(")", 1)[1].split() if tok.isdigit()]
+                    return numbers[2]          # fetch KiB, write KiB, scaled bytes, algorithmic
+    except (OSError, IndexError, ValueError):
+        pass
+    return None
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="comma list of configs to time (c1,c2,c3,c4,c5,extra,apps); "
                     "c2 is always timed; 'extra' adds LayerNorm backward and the other GEMM layouts and element "
@@ -62,11 +81,21 @@ def main():
         return not only or name in only
 
     def timed(fn, steps=K, warmup=W):
-        """Average milliseconds per call over ``steps`` calls, bracketed by synchronisation."""
-        for _ in range(warmup):
-            fn()
-        torch.cuda.synchronize()
+        """Average milliseconds per call over exactly ``steps`` calls timed with events on the launch
+        stream.  Untimed before them: ``warmup`` calls, then as many more as fill SETTLE_MS of device
+        time, queued back to back with the timed ones -- after an idle gap the part needs about 20 ms
+        of continuous work to return to its steady clocks (a launch of the row softmax reads 4.3 TB/s
+        in the first 2 ms after a gap, 5.8 after 10 ms and 6.15 from 25 ms on)."""
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(max(1, warmup)):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        per_call = start.elapsed_time(stop) / max(1, warmup)
+        for _ in range(min(5000, int(SETTLE_MS / max(per_call, 1e-3)) + 1)):
+            fn()
         start.record()
         for _ in range(steps):
             fn()
@@ -84,6 +113,18 @@ def main():
             call(sets[state["i"] % n])
             state["i"] += 1
         return timed(fn)
+
+    cpu_threads = torch.get_num_threads()
+
+    def cpu_timed(fn, unit_count, unit, sample):
+        """One timed run of a CPU-path function: a ``cpu_baseline`` entry (None with --skip-cpu)."""
+        if ns.skip_cpu:
+            return None
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        return dict(value=unit_count / dt / 1e9, unit=unit, cores=cpu_threads, kind="port",
+                    sample=f"{sample}; {dt:.2f} s, one run, {cpu_threads} threads of {os.cpu_count()} visible cores")
 
     kernels = {}
     gen = lambda seed: torch.Generator().manual_seed(seed)  # noqa: E731
@@ -134,6 +175,18 @@ def main():
                                                 frac_hbm=b1 / rot / 1e6 / HBM_PEAK_GBS, bytes=b1,
                                                 parity="bit-exact",
                                                 note="gbs = rotating buffers (1 GiB pool); gbs_hot = cache resident")
+        if not ns.skip_cpu:
+            from lego_amd.kernels.transpose import python_offsets
+            from oracle import cpu_path
+            s1, d1 = python_offsets(32, 32)
+            x1c = x1.cpu()
+            got1 = {}
+            kernels["c1_transpose_f32_4096"]["cpu_baseline"] = cpu_timed(
+                lambda: got1.update(y=cpu_path.transpose_printed(x1c, s1, d1, 32, 32)), b1, "GB/s",
+                "the whole 4096x4096 fp32 matrix: printed offsets of both TileBy([128,128],[32,32]) layouts "
+                "evaluated with torch.arange, then one gather/scatter")
+            assert torch.equal(got1["y"], ops.transpose(x1).cpu()), "GPU result differs from the CPU path"
+            del x1c, got1
         del x1, y1
 
     # ---- C3: softmax and LayerNorm forward, fp16 8192x8192 -------------------------------------
@@ -170,6 +223,13 @@ def main():
                                  frac_hbm=by3 / rot / 1e6 / HBM_PEAK_GBS, bytes=by3, max_abs_err_vs_fp32=err,
                                  note="gbs = rotating buffers (1 GiB pool); gbs_hot = cache resident; "
                                       "x ~ N(0, sigma=2)")
+        if not ns.skip_cpu:
+            from oracle import kernels as ok3
+            kernels["c3_softmax_f16_8192"]["cpu_baseline"] = cpu_timed(
+                lambda: ok3.softmax(x3c), by3, "GB/s", "the whole 8192x8192 matrix: torch.softmax(x.float(), -1).half()")
+            kernels["c3_layernorm_fwd_f16_8192"]["cpu_baseline"] = cpu_timed(
+                lambda: ok3.layernorm_fwd(x3c, w3c, b3c, 1e-5), by3, "GB/s",
+                "the whole 8192x8192 matrix: F.layer_norm(x.float(), ...).half() plus mean and rstd")
         # next row: LayerNorm backward (reference formula: 3 * numel * element size, layernorm.py:555)
         if want("extra"):
             dy3 = (0.1 * torch.randn(m3, n3, generator=gen(6))).half().to(dev)
@@ -226,6 +286,13 @@ def main():
                                            vendor_library_tflops_b_moved_128_bytes=fl4 / lib_ms_s / 1e9,
                                            note="vendor_library = torch.matmul (hipBLASLt) on the same buffers")
         del b4s, b4s_buf
+        if not ns.skip_cpu:
+            from oracle import kernels as ok4
+            a4c, b4c = a4[:1024].cpu(), b4.cpu()
+            kernels["c4_gemm_f16_8192"]["cpu_baseline"] = cpu_timed(
+                lambda: ok4.gemm(a4c, b4c), 2 * 1024 * n4 * n4 / 1e3, "TFLOP/s",
+                "rows 0..1023 of A (an eighth of the workload): (A.float() @ B.float()).half()")
+            del a4c, b4c
         if want("extra"):
             for ta, tb in ((0, 1), (1, 0), (1, 1)):
                 def gv(ta=ta, tb=tb):
@@ -283,6 +350,16 @@ def main():
         ms = timed(gg, steps=max(5, K // 5), warmup=max(2, W // 5))
         kernels["c5_grouped_gemm_f16"] = dict(ms=ms, tflops=fl5 / ms / 1e9, frac_mfma=fl5 / ms / 1e9 / MFMA_F16_PEAK_TFLOPS,
                                               flop=fl5, problems=dims, rel_err_vs_fp32=rel)
+        plan5 = (ctypes.c_int * 3)()
+        runtime.call("lego_hip_grouped_gemm_f16_plan", sz, 8, plan5)
+        kernels["c5_grouped_gemm_f16"]["launch"] = dict(tile=plan5[0], tiles=plan5[1], tiles_split_in_halves=plan5[2])
+        if not ns.skip_cpu:
+            from oracle import kernels as ok5
+            Ac, Bc = [t.cpu() for t in A], [t.cpu() for t in B]
+            kernels["c5_grouped_gemm_f16"]["cpu_baseline"] = cpu_timed(
+                lambda: ok5.grouped_gemm(Ac, Bc), fl5 / 1e3, "TFLOP/s",
+                "all 8 problems: (A.float() @ B.float()).half() each")
+            del Ac, Bc
         del A, B, C
 
     # ---- next rows: the reference's lego_c benchmark programs (stencils on bricks, Needleman-Wunsch, LUD) ----
@@ -329,23 +406,25 @@ def main():
                                                  note="time of a matrix copy subtracted; block steps of 64 in pairs")
             del a0, wk
 
-    # ---- CPU baseline: the oracle on a bounded panel of the headline matrix ------------------------------
+    # ---- CPU baseline: the reference's CPU path on a bounded panel of the headline matrix -----------------
     cpu = None
     if not ns.skip_cpu:
-        from oracle import kernels as ok
+        from lego_amd.kernels.transpose import python_offsets
+        from oracle import cpu_path
         rows = 8192
         c2()                      # y2 was last written by the copy ceiling measurement
         torch.cuda.synchronize()
         panel = x2[:rows].cpu()
-        torch.set_num_threads(1)       # a scalar port: numpy's index arithmetic is single-threaded anyway
+        src_text, dst_text = python_offsets(64, 64)
         t0 = time.perf_counter()
-        got = ok.transpose(panel, 64, 64)
+        got = cpu_path.transpose_printed(panel, src_text, dst_text, 64, 64, total_rows=n2)
         dt = time.perf_counter() - t0
-        assert torch.equal(got, y2[:, :rows].cpu()), "GPU result differs from the CPU oracle"
-        cpu = dict(value=2 * panel.numel() * 2 / dt / 1e9, unit="GB/s", cores=1, kind="port",
-                   sample=f"rows 0..{rows - 1} of the 16384x16384 fp16 matrix ({rows}x16384 panel, "
-                          f"{rows}/16384 of the workload): offsets of both LEGO layouts evaluated with numpy, then one "
-                          f"gather/scatter; {dt:.2f} s on one of {os.cpu_count()} visible cores")
+        assert torch.equal(got, y2[:, :rows].cpu()), "GPU result differs from the CPU path"
+        cpu = dict(value=2 * panel.numel() * 2 / dt / 1e9, unit="GB/s", cores=cpu_threads, kind="port",
+                   sample=f"rows 0..{rows - 1} of the 16384x16384 fp16 matrix ({rows}/16384 of the workload): the "
+                          f"offsets of both LEGO layouts as the Python/Triton printer emits them, evaluated with "
+                          f"torch.arange for tl.arange, then one gather/scatter; {dt:.2f} s, one run, "
+                          f"{cpu_threads} threads of {os.cpu_count()} visible cores")
 
     line = {
         "metric": "HBM GB/s (transpose/softmax/LN) + fp16 GEMM TFLOPS, % of roofline, 1 GPU",
@@ -355,8 +434,8 @@ def main():
                                "column-major, 1x4 tiles per workgroup, workgroups in windows of 128x8 macro tiles, XOR-swizzled LDS "
                                "staging, inputs N(0,1) seed 1"},
         "roofline": {"bound": "hbm", "achieved": gbs2, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gbs2 / HBM_PEAK_GBS, "traffic": HEADLINE_TRAFFIC_BYTES,
-                     "kernel": "lego_transpose_f16_64x256_w128x8", "algorithmic_bytes_per_launch": bytes2},
+                     "frac": gbs2 / HBM_PEAK_GBS, "traffic": headline_traffic_bytes(),
+                     "kernel": HEADLINE_KERNEL, "algorithmic_bytes_per_launch": bytes2},
         "cpu_baseline": cpu,
         "kernels": kernels,
         "peaks": {"hbm_gbs": HBM_PEAK_GBS, "mfma_f16_tflops": MFMA_F16_PEAK_TFLOPS,

@@ -182,7 +182,7 @@ int lego_hip_grouped_gemm_f16_split(const void* const* a, const void* const* b, 
                                     const int* sizes3, int groups, int split_tiles, void* stream);
 
 /* Tuning entry points: as above, with the launch shape chosen by the caller
- * (waves_per_row in {1, 2, 4, 16}; N a multiple of 8 and at most 8192 * waves_per_row, 16384 for 4).  Used by the benchmark to compare variants. */
+ * (waves_per_row in {1, 2, 4, 8, 16}; N a multiple of 8 and at most 8192 * waves_per_row, 16384 for 4 and 8).  Used by the benchmark to compare variants. */
 int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per_row, void* stream);
 int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const void* b,
                                    float* mean, float* rstd, int M, int N, float eps,

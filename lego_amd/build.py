@@ -39,12 +39,15 @@ TRANSPOSE = {
 }
 # (element type, vectorised, waves per row): 16-byte accesses need N % (16/size) == 0; the
 # element-per-access kernels ("s") take any N
-ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f32", True, 1), ("f32", True, 4),
+ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f16", True, 8), ("f32", True, 1), ("f32", True, 4),
            ("f16", False, 1), ("f32", False, 1), ("f16", False, 4), ("f32", False, 4),
            ("f16", True, 16), ("f32", True, 16), ("f16", False, 16), ("f32", False, 16),
            ("bf16", True, 1), ("bf16", True, 4), ("bf16", True, 16), ("bf16", False, 1), ("bf16", False, 4),
            ("bf16", False, 16)]
+# LayerNorm launches of many rows: this many workgroups that stage gamma and beta in LDS and walk the rows
+ROWWISE_STREAM_WGS = {("f16", True, 8): 512}
 ROWWISE_DEFAULT_WAVES = 4
+ROWWISE_WIDE_TEAM_ABOVE_N, ROWWISE_WIDE_TEAM_FROM_M = 6144, 4096
 ROWWISE_MAX_N = rowwise.MAX_N
 GEMM = dict(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8)
 GEMM_SMALL_TILE = 128
@@ -70,7 +73,7 @@ def generate():
             units.append(unit)
             tmeta.setdefault(dtype, []).append(meta)
     units.append(transpose.emit_any())
-    units += [rowwise.emit(w, dtype, vec) for dtype, vec, w in ROWWISE]
+    units += [rowwise.emit(w, dtype, vec, stream_wgs=ROWWISE_STREAM_WGS.get((dtype, vec, w), 0)) for dtype, vec, w in ROWWISE]
     units.append(rowwise.emit_long())
     for dtype in GEMM_DTYPES:
         for ta in (False, True):
@@ -124,7 +127,11 @@ def generate():
           "// register footprint of long rows small enough for full occupancy, sixteen (a whole",
           "// workgroup of 1024 lanes) hold the rows that four cannot",
           f"inline int lego_rowwise_default_wpr(int n) {{ return n <= 2048 ? 1 : n <= {rowwise.MAX_N_SMALL_TEAMS} ? "
-          f"{ROWWISE_DEFAULT_WAVES} : {rowwise.LONG_ROW_WAVES}; }}", ""]
+          f"{ROWWISE_DEFAULT_WAVES} : {rowwise.LONG_ROW_WAVES}; }}",
+          "// fp16 rows of whole vectors: eight waves (a workgroup of 512 lanes, two to four vectors per lane) for long",
+          "// rows of tall matrices, where they measure 3-5 % above four waves; fewer rows leave too few workgroups",
+          f"inline int lego_rowwise_f16_wpr(int m, int n) {{ return n > {ROWWISE_WIDE_TEAM_ABOVE_N} && n <= "
+          f"{rowwise.MAX_N_SMALL_TEAMS} && m >= {ROWWISE_WIDE_TEAM_FROM_M} ? 8 : lego_rowwise_default_wpr(n); }}", ""]
     h += ["unsigned lego_layernorm_bwd_groups(int M, int N);", "unsigned lego_layernorm_bwd_f32_groups(int M, int N);",
           "unsigned lego_layernorm_bwd_bf16_groups(int M, int N);",
           "hipError_t lego_layernorm_bwd_f32_launch(const void*, const void*, const void*, const float*, const float*, "

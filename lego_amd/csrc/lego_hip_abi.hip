@@ -98,6 +98,7 @@ int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per
     case 1: return ok_or(lego_softmax_f16_w1_launch(x, y, M, N, as_stream(stream)));
     case 2: return ok_or(lego_softmax_f16_w2_launch(x, y, M, N, as_stream(stream)));
     case 4: return ok_or(lego_softmax_f16_w4_launch(x, y, M, N, as_stream(stream)));
+    case 8: return ok_or(lego_softmax_f16_w8_launch(x, y, M, N, as_stream(stream)));
     case 16: return ok_or(lego_softmax_f16_w16_launch(x, y, M, N, as_stream(stream)));
     default: return kInvalid;
   }
@@ -112,7 +113,7 @@ int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream)
     return ok_or((long_row ? lego_softmax_f16s_w16_launch : lego_rowwise_default_wpr(N) == 1 ? lego_softmax_f16s_w1_launch
                                                                                            : lego_softmax_f16s_w4_launch)(
         x, y, M, N, as_stream(stream)));
-  return lego_hip_softmax_f16_wpr(x, y, M, N, lego_rowwise_default_wpr(N), stream);
+  return lego_hip_softmax_f16_wpr(x, y, M, N, lego_rowwise_f16_wpr(M, N), stream);
 }
 
 int lego_hip_softmax_f32(const void* x, void* y, int M, int N, void* stream)
@@ -137,6 +138,7 @@ int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const 
     case 1: return ok_or(lego_layernorm_fwd_f16_w1_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
     case 2: return ok_or(lego_layernorm_fwd_f16_w2_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
     case 4: return ok_or(lego_layernorm_fwd_f16_w4_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+    case 8: return ok_or(lego_layernorm_fwd_f16_w8_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
     case 16: return ok_or(lego_layernorm_fwd_f16_w16_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
     default: return kInvalid;
   }
@@ -152,7 +154,7 @@ int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void
     return ok_or((long_row ? lego_layernorm_fwd_f16s_w16_launch : lego_rowwise_default_wpr(N) == 1 ? lego_layernorm_fwd_f16s_w1_launch
                                                                                                  : lego_layernorm_fwd_f16s_w4_launch)(
         x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
-  return lego_hip_layernorm_fwd_f16_wpr(x, y, w, b, mean, rstd, M, N, eps, lego_rowwise_default_wpr(N), stream);
+  return lego_hip_layernorm_fwd_f16_wpr(x, y, w, b, mean, rstd, M, N, eps, lego_rowwise_f16_wpr(M, N), stream);
 }
 
 int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void* b,

@@ -27,7 +27,7 @@ LONG_ROW_WAVES = 16
 VPTS = (1, 2, 4, 8, 16, 32, 64)
 
 
-def emit(waves_per_row=1, dtype="f16", vectorised=True):
+def emit(waves_per_row=1, dtype="f16", vectorised=True, seq_max_wpr=4, prefetch_max_wpr=4, stream_wgs=0):
     """One translation unit: every register footprint ``V`` of one (waves per row, element type,
     access width) combination.  ``vectorised=False`` emits the kernels that take rows of any length
     and alignment (the reference's own softmax test is 1823 x 781): the elements before a row's
@@ -56,11 +56,18 @@ def emit(waves_per_row=1, dtype="f16", vectorised=True):
     row_base = tidy(X[row, 0, 0, 0], {row: (0, M)})
     vec_off = tidy(X[0, v, 0, 0], {v: (0, N / EPV)})
     stat = OrderBy(Row(M)).TileBy([M])[row,]
+    # many rows per workgroup (LayerNorm with gamma and beta staged in LDS): workgroup wg of G walks rows
+    # Row(STEPS, G)[step, wg]
+    G, STEPS, step = size("G"), size("STEPS"), idx("step")
+    stream_row = tidy(OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])[step, wg], {step: (0, STEPS), wg: (0, G)})
 
     params = dict(
         banner=BANNER, WPR=WPR, TEAM=TEAM, RPW=RPW, THREADS=threads,
         VPTS=[vp for vp in VPTS if vp * EPV <= 128 and lo < vp * TEAM * EPV <= hi],
         dtype=dtype, elt=elt, EPV=EPV, ESIZE=esize, RAGGED=not vectorised, tag=tag,
+        SEQ_MAX_WPR=seq_max_wpr, PREFETCH_MAX_WPR=prefetch_max_wpr,
+        STREAM=vectorised and RPW == 1 and WPR < LONG_ROW_WAVES and stream_wgs > 0, STREAM_WGS=stream_wgs,
+        stream_layout="OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])[step, wg]", stream_row=code(stream_row),
         row_layout=f"OrderBy(Row(NWG, {RPW})).TileBy([NWG], [{RPW}])[wg, team]",
         lane_layout=f"OrderBy(Row({RPW}, {TEAM})).TileBy([{RPW}, {TEAM}]).inv(t); vector = it*{TEAM} + lane",
         x_layout=f"OrderBy(Row(M, N)).TileBy([M, N/{EPV}], [1, {EPV}])[row, v, 0, :]",

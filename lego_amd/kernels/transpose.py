@@ -231,3 +231,21 @@ def emit_any():
                   tx=code(tidy(tx_e, {t: (0, 256)})), ty=code(tidy(ty_e, {t: (0, 256)})))
     text = template("transpose_any.hip.j2").render(**params)
     return Emitted("transpose_any.hip", text, ["lego_transpose_any_launch"])
+
+
+def python_offsets(tile_r, tile_c):
+    """The transpose as the reference's Python/Triton backend states it: the printed offsets of logical
+    index ``(bi, bj, i, j)`` in the row-major source ``OrderBy(Row(R, C)).TileBy([R/TR, C/TC], [TR, TC])``
+    and in the column-major destination with the same tiling, every index a whole axis
+    (``tl.arange(...)`` broadcast along its own axis of a rank-4 block).  Evaluated with
+    ``torch.arange`` standing for ``tl.arange`` this text is LEGO's CPU index path
+    (lego/lego_python.py:5-37); ``nbi`` and ``nbj`` are the numbers of tile rows and columns taken."""
+    from ..lego import TritonRange, get_arange
+    from ..lego_python import LEGOPythonCodePrinter
+    R, C, nbi, nbj = size("R"), size("C"), size("nbi"), size("nbj")
+    axes = [TritonRange(get_arange(0, n), a, 4) for a, n in enumerate((nbi, nbj, tile_r, tile_c))]
+    levels = ([R / tile_r, C / tile_c], [tile_r, tile_c])
+    printer = LEGOPythonCodePrinter(allow_unknown_functions=True)
+    src = OrderBy(Row(R, C)).TileBy(*levels)[tuple(axes)]
+    dst = OrderBy(Col(R, C)).TileBy(*levels)[tuple(axes)]
+    return printer.doprint(sp.simplify(src)), printer.doprint(sp.simplify(dst))

@@ -64,6 +64,20 @@ def layernorm_fwd(x, weight, bias, eps=1e-5):
     return y.to(x.dtype), mean, rstd
 
 
+def layernorm_fwd_unrounded(x, weight, bias, eps=1e-5):
+    """``y`` of :func:`layernorm_fwd` in fp32, before it is rounded to the tensors' type (what the
+    reference's kernel holds in registers before its store, layernorm.py:94-101)."""
+    return torch.nn.functional.layer_norm(x.float(), (x.shape[-1],), weight.float(), bias.float(), eps)
+
+
+def half_spacing(y32: torch.Tensor, dtype) -> torch.Tensor:
+    """Half the distance between neighbouring ``dtype`` values around each fp32 value: what a
+    correctly rounded ``dtype`` result may differ from the fp32 value by."""
+    bits, emin = {torch.float16: (10, -14), torch.bfloat16: (7, -126)}[dtype]
+    expo = torch.floor(torch.log2(y32.abs().clamp(min=2.0 ** emin)))
+    return torch.exp2(expo - bits - 1)
+
+
 def gemm(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     return (a.float() @ b.float()).to(a.dtype)
 

@@ -1,0 +1,48 @@
+"""The CPU baseline's path: offsets printed by the Python/Triton printer, evaluated with torch.arange,
+against the oracle's integer layouts and the textbook transpose; and the benchmark's reading of the
+committed HBM-traffic summary."""
+import numpy as np
+import pytest
+import torch
+
+from lego_amd.kernels.transpose import python_offsets
+from oracle import cpu_path
+from oracle import kernels as ok
+from oracle import lego_index as li
+
+
+@pytest.mark.parametrize("rows,cols,tr,tc", [(256, 384, 64, 64), (128, 128, 32, 32), (96, 160, 32, 16)])
+def test_printed_offsets_are_the_oracle_layouts(rows, cols, tr, tc):
+    src_text, dst_text = python_offsets(tr, tc)
+    names = dict(R=rows, C=cols, nbi=rows // tr, nbj=cols // tc)
+    src, dst = ok.transpose_layouts(rows, cols, tr, tc)
+    assert np.array_equal(cpu_path.evaluate(src_text, **names).numpy(), np.array(src.offsets()))
+    assert np.array_equal(cpu_path.evaluate(dst_text, **names).numpy(), np.array(dst.offsets()))
+    # closed forms of the two layouts: r*C + c and c*R + r
+    bi, bj, i, j = np.meshgrid(np.arange(rows // tr), np.arange(cols // tc), np.arange(tr), np.arange(tc), indexing="ij")
+    assert np.array_equal(cpu_path.evaluate(src_text, **names).numpy(), (bi * tr + i) * cols + bj * tc + j)
+    assert np.array_equal(cpu_path.evaluate(dst_text, **names).numpy(), (bj * tc + j) * rows + bi * tr + i)
+
+
+def test_cpu_path_transposes_whole_matrices_and_panels():
+    g = torch.Generator().manual_seed(0)
+    src_text, dst_text = python_offsets(64, 64)
+    x = torch.randn(256, 384, generator=g).half()
+    assert torch.equal(cpu_path.transpose_printed(x, src_text, dst_text, 64, 64), x.t().contiguous())
+    assert torch.equal(cpu_path.transpose_printed(x, src_text, dst_text, 64, 64), ok.transpose(x, 64, 64))
+    got = cpu_path.transpose_printed(x[:128], src_text, dst_text, 64, 64, total_rows=256)
+    assert torch.equal(got, x.t()[:, :128].contiguous())
+
+
+def test_benchmark_reads_the_committed_traffic_summary():
+    import bench
+    got = bench.headline_traffic_bytes()
+    text = open(bench.TRAFFIC_PROFILE).read()
+    row = next(line for line in text.splitlines() if line.startswith(bench.HEADLINE_KERNEL + " "))
+    fetch_kib, write_kib, scaled, algorithmic = [int(t) for t in row.split(")", 1)[1].split()[:4]]
+    assert got == scaled
+    # the scaled figure is what the counters say: FETCH_SIZE counts half of every 128-byte request at
+    # this access width (the copy calibration in the same file reads 262150 KiB for 512 MiB: factor
+    # 2 * 262144 / 262150), WRITE_SIZE all of it
+    assert abs(scaled - (2.0 * 262144 / 262150 * fetch_kib + write_kib) * 1024) <= 4096
+    assert algorithmic == 2 * 16384 * 16384 * 2

@@ -126,11 +126,28 @@ def test_transpose_rejects_bad_arguments(ops):
 TOL = 2e-3
 
 
-@pytest.mark.parametrize("wpr", [None, 1, 2, 4])
-@pytest.mark.parametrize("M,N", [(7, 8), (33, 520), (64, 1024), (5, 2048), (129, 4096), (16, 8192), (3, 16384)])
+def _assert_layernorm_forward(y, x, w, b, eps=1e-5):
+    """A 16-bit LayerNorm result against the un-rounded fp32 oracle.  The contract is on the fp32
+    arithmetic (max abs err <= 2e-3 after fp32 accumulation); the store then rounds to 16 bits, which
+    moves a value by up to half a spacing (2^-10 for fp16 values in [2, 4)).  So: the result is within
+    half a spacing of the fp32 oracle, plus 1e-4 for the fp32 arithmetic itself (summation order), and
+    wherever |y| < 2 the literal bound holds against the rounded oracle as well."""
+    ref32 = ok.layernorm_fwd_unrounded(x, w, b, eps)
+    err = (y.cpu().float() - ref32).abs()
+    slack = ok.half_spacing(ref32, x.dtype) + 1e-4
+    worst = (err - slack).max().item()
+    assert worst <= 0, f"{worst:.3e} beyond half a spacing + 1e-4"
+    small = ref32.abs() < 2
+    if x.dtype == torch.float16 and small.any():
+        assert (y.cpu().float() - ref32.to(x.dtype).float()).abs()[small].max().item() <= TOL
+
+
+@pytest.mark.parametrize("wpr", [None, 1, 2, 4, 8])
+@pytest.mark.parametrize("M,N", [(7, 8), (33, 520), (64, 1024), (5, 2048), (129, 4096), (16, 8192), (3, 16384),
+                                 (4100, 8200)])     # tall and long: the default takes teams of eight waves
 def test_softmax_matches_oracle(ops, M, N, wpr):
     print(f"softmax {M}x{N} wpr={wpr}", flush=True)
-    if wpr is not None and N > 8192 * wpr:
+    if wpr is not None and N > min(8192 * wpr, 16384):
         from lego_amd.runtime import LegoHipError
         with pytest.raises(LegoHipError):      # a row must fit the registers of its team
             ops.softmax(torch.zeros(M, N, device="cuda", dtype=torch.half), waves_per_row=wpr)
@@ -195,8 +212,10 @@ def test_layernorm_ragged_and_fp32(ops, dtype, M, N):
     b = (0.1 * torch.randn(N, generator=g)).to(dtype)
     want_y, want_mean, want_rstd = ok.layernorm_fwd(x, w, b, 1e-5)
     y, mean, rstd = ops.layer_norm_fwd(x.cuda(), w.cuda(), b.cuda(), 1e-5)
-    tol = 2 * TOL if dtype == torch.float16 else 2e-5
-    assert (y.cpu().float() - want_y.float()).abs().max().item() <= tol
+    if dtype == torch.float16:
+        _assert_layernorm_forward(y, x, w, b)
+    else:
+        assert (y.cpu().float() - want_y.float()).abs().max().item() <= 2e-5
     assert torch.allclose(mean.cpu(), want_mean, atol=1e-4, rtol=1e-4)
     if N > 1:
         assert torch.allclose(rstd.cpu(), want_rstd, atol=1e-4, rtol=1e-3)
@@ -226,11 +245,13 @@ def test_layernorm_fp32_long_rows_through_the_c_abi(ops, N):
     assert torch.allclose(rstd.cpu(), want_rstd, atol=1e-4, rtol=1e-3)
 
 
-@pytest.mark.parametrize("wpr", [None, 1, 2, 4])
-@pytest.mark.parametrize("M,N", [(7, 8), (33, 520), (64, 1024), (129, 4096), (1151, 8192), (3, 16384)])
+@pytest.mark.parametrize("wpr", [None, 1, 2, 4, 8])
+# 1151 and 4100 rows with eight waves: workgroups that stage gamma and beta in LDS and walk two to nine rows each
+@pytest.mark.parametrize("M,N", [(7, 8), (33, 520), (64, 1024), (129, 4096), (1151, 8192), (3, 16384), (4100, 8200),
+                                 (1030, 16384)])
 def test_layernorm_matches_oracle(ops, M, N, wpr):
     print(f"layernorm {M}x{N} wpr={wpr}", flush=True)
-    if wpr is not None and N > 8192 * wpr:
+    if wpr is not None and N > min(8192 * wpr, 16384):
         pytest.skip("a row must fit the registers of its team")
     g = _gen(3)
     x = (2.0 * torch.randn(M, N, generator=g)).half()
@@ -238,9 +259,7 @@ def test_layernorm_matches_oracle(ops, M, N, wpr):
     b = (0.1 * torch.randn(N, generator=g)).half()
     want_y, want_mean, want_rstd = ok.layernorm_fwd(x, w, b, 1e-5)
     y, mean, rstd = ops.layer_norm_fwd(x.cuda(), w.cuda(), b.cuda(), 1e-5, waves_per_row=wpr)
-    # y is fp16 with magnitude up to ~6: half an ulp there is 2e-3, so compare before the final
-    # rounding as well (the tolerance of the contract is on the value, not on the rounding)
-    assert (y.cpu().float() - want_y.float()).abs().max().item() <= 2 * TOL
+    _assert_layernorm_forward(y, x, w, b)
     assert torch.allclose(mean.cpu(), want_mean, atol=1e-4, rtol=1e-4)
     assert torch.allclose(rstd.cpu(), want_rstd, atol=1e-4, rtol=1e-4)
 
@@ -256,7 +275,7 @@ def test_layernorm_reference_test_shape(ops):
     from lego_amd.ops import lego_layer_norm
     got = lego_layer_norm(x.cuda(), (8192,), w.cuda(), b.cuda(), 1e-5).cpu()
     assert torch.allclose(got.float(), want.float(), atol=1e-2, rtol=0)
-    assert (got.float() - want.float()).abs().max().item() <= TOL
+    _assert_layernorm_forward(got, x, w, b)
 
 
 def test_layernorm_backward_reference_test(ops):
@@ -354,7 +373,7 @@ def test_layernorm_bfloat16_forward_and_backward(ops, M, N):
     yr = torch.nn.functional.layer_norm(xc, (N,), wc, bc, 1e-5)
     yr.backward(dy.float())
     # results are rounded to bfloat16: half a spacing relative to the magnitude, 2^-9
-    assert ((y.detach().cpu().float() - yr.detach()).abs() <= 2.0 ** -8 * yr.detach().abs() + 1e-3).all()
+    _assert_layernorm_forward(y.detach(), x, w, b)
     assert ((xd.grad.cpu().float() - xc.grad).abs() <= 2.0 ** -8 * xc.grad.abs() + 1e-3).all()
     assert ((wd.grad.cpu().float() - wc.grad).abs() <= 2.0 ** -8 * wc.grad.abs() + 2e-3 * max(1.0, wc.grad.abs().max().item())).all()
     assert ((bd.grad.cpu().float() - bc.grad).abs() <= 2.0 ** -8 * bc.grad.abs() + 2e-3 * max(1.0, bc.grad.abs().max().item())).all()
@@ -372,11 +391,7 @@ def test_config3_full_size(ops):
     assert (s.float() - ok.softmax(x).float()).abs().max().item() <= TOL
     y, mean, rstd = ops.layer_norm_fwd(xd, w.cuda(), b.cuda(), 1e-5)
     want_y, want_mean, want_rstd = ok.layernorm_fwd(x, w, b, 1e-5)
-    err = (y.cpu().float() - want_y.float()).abs()
-    # fp16 spacing is 2^-9 = 1.95e-3 for |y| in [2,4) and 3.9e-3 in [4,8): a correctly rounded
-    # result can differ from another correctly rounded result by one spacing
-    assert err[want_y.float().abs() < 2].max().item() <= TOL
-    assert (err <= want_y.float().abs().clamp(min=1) * 2 ** -9).all()
+    _assert_layernorm_forward(y, x, w, b)
     assert torch.allclose(mean.cpu(), want_mean, atol=1e-4, rtol=1e-4)
 
 
