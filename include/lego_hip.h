@@ -7,7 +7,9 @@
  *   - all tensor pointers are BORROWED DEVICE pointers, 16-byte aligned, row-major and
  *     contiguous; nothing is allocated, freed or synchronised: the kernel is enqueued on
  *     `stream` (a hipStream_t; NULL = the default stream) and the call returns;
- *   - stateless and re-entrant: safe from several host threads on distinct streams.
+ *   - re-entrant: safe from several host threads on distinct streams.  Two entry points keep state between
+ *     calls, both described where they are declared: lego_hip_lud_f32 (a side stream per caller's stream) and
+ *     lego_hip_layernorm_bwd_f16_noalloc (a built-in scratch array per device).
  *
  * The reference has no FFI: its kernels are reached through generated Python host
  * functions.  Each entry point below names the reference host function it stands behind.
@@ -136,9 +138,14 @@ int lego_hip_stencil_laplacian_f32(const float* in, float* out, const float* c, 
  * strict lower triangle holds L (unit diagonal implied) and the upper triangle holds U, as
  * Rodinia's lud (the reference's thread-coarsening benchmark: benchmarks/cuda/lud.py:5-12,
  * kernels lud/lud_kernel_temp.cu:14-352, host loop :358-390).  n a multiple of 64, at most 32768.
- * From n = 4928 on, part of the work is enqueued on a second stream that the library creates on the
- * first such call on a device and keeps until the process ends; it is forked from and joined back
- * into `stream` with events inside the call, so the caller sees ordinary stream order. */
+ * From n = 4928 on, part of the work is enqueued on a second stream, forked from and joined back into
+ * `stream` with events inside the call, so the caller sees ordinary stream order (captured into a graph,
+ * the fork and join become graph edges).  The library makes that stream and its two events on the first
+ * such call for a given (device, `stream`) pair -- the device of `stream` must be current -- and keeps
+ * them until the process ends: callers on distinct streams share nothing.  After 32 such pairs, and for a
+ * `stream` that is under capture the first time it is seen (nothing is created during a capture), the
+ * call stays on `stream` alone (same results, less overlap).  Concurrent calls on the SAME `stream` from
+ * several threads are not supported, as for any stream-ordered work. */
 int lego_hip_lud_f32(float* m, int n, void* stream);
 
 /* The launches that lego_hip_lud_f32 enqueues for an n x n matrix, in order, without touching a device: six

@@ -116,6 +116,12 @@ def layer_norm_bwd(dy, x, weight, mean, rstd):
     _check(dy_arg, x.dtype, "dy")
     _check(weight, x.dtype, "weight", ndim=1)
     M, N = x_arg.shape
+    if dy_arg.shape != x_arg.shape or weight.shape[0] != N:
+        raise ValueError("dy must have the shape of x and weight the length of its rows")
+    for name, stat in (("mean", mean), ("rstd", rstd)):
+        _check(stat, torch.float32, name, ndim=1)       # the forward pass's fp32 statistics, one per row
+        if stat.shape[0] != M or stat.device != x.device:
+            raise ValueError(f"{name} must hold one float32 per row of x, on its device")
     need = ctypes.c_ulonglong(0)
     runtime.call("lego_hip_layernorm_bwd_workspace_bytes" if tag == "f16" else f"lego_hip_layernorm_bwd_{tag}_workspace_bytes",
                  M, N, ctypes.byref(need))
@@ -235,7 +241,14 @@ def _stencil(entry, x, c, radius, bricks, out):
     n = x.shape[0]
     if x.shape != (n, n, n):
         raise ValueError("x must be a cube")
-    out = torch.zeros_like(x) if out is None else out
+    if out is None:
+        out = torch.zeros_like(x)
+    else:
+        _check(out, torch.float32, "out", ndim=3)
+        if out.shape != x.shape or out.device != x.device:
+            raise ValueError("out must have the shape and device of x")
+        if out.data_ptr() == x.data_ptr():
+            raise ValueError("out must not alias x")
     runtime.call(entry, _ptr(x), _ptr(out), _ptr(c), n, int(radius), 1 if bricks else 0, _stream())
     return out
 

@@ -326,6 +326,20 @@ def test_layernorm_backward_matches_oracle(ops, M, N):
     assert (db.cpu().float() - bc.grad).abs().max().item() <= 2e-3 * max(1.0, bc.grad.abs().max().item())
 
 
+def test_layernorm_backward_rejects_foreign_statistics(ops):
+    """mean and rstd reach the kernel as raw pointers: anything but one float32 per row on the device is refused."""
+    print("layernorm backward argument checks", flush=True)
+    x = torch.zeros(4, 64, dtype=torch.half, device="cuda")
+    w = torch.ones(64, dtype=torch.half, device="cuda")
+    good = torch.zeros(4, device="cuda")
+    for mean, rstd in ((good.cpu(), good), (good, good.half()), (good[:3], good), (good, torch.zeros(8, device="cuda")[::2]),
+                       (good.view(2, 2), good)):
+        with pytest.raises(ValueError):
+            ops.layer_norm_bwd(x, x, w, mean, rstd)
+    with pytest.raises(ValueError):
+        ops.layer_norm_bwd(torch.zeros(4, 32, dtype=torch.half, device="cuda"), x, w, good, good)
+
+
 @pytest.mark.parametrize("M,N", [(1, 4), (7, 5), (300, 1000), (129, 4096), (33, 4099), (40, 16384)])
 def test_layernorm_backward_fp32(ops, M, N):
     """fp32 tensors through the autograd wrapper, against fp64 autograd on the CPU."""

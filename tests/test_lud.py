@@ -213,9 +213,10 @@ def test_gpu_large_matrix_reproduces_its_factors(n):
 
 @pytest.mark.gpu
 def test_gpu_call_with_second_stream_replays_from_a_hip_graph():
-    """At n = 8256 the call forks to the library's second stream and joins it back with events; captured into a
-    graph (after an eager call, which creates that stream), every replay gives the bits of the eager result, with
-    eager work and synchronisation between the replays."""
+    """At n = 8256 the call forks to a second stream of the library and joins it back with events; captured into a
+    graph on a stream that an eager call has used before (which made that stream's side stream), every replay
+    gives the bits of the eager result, with eager work and synchronisation between the replays.  Captured on a
+    stream the library has never seen, the call creates nothing and stays on the one stream: same bits."""
     from lego_amd import ops
     print("lud n=8256 captured into a graph", flush=True)
     n = 8256
@@ -232,14 +233,16 @@ def test_gpu_call_with_second_stream_replays_from_a_hip_graph():
         ops.lud(w)                       # warm-up on a side stream, outside the capture
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        ops.lud(w)
-    for trial in range(3):
-        w.copy_(a)
-        graph.replay()
-        torch.cuda.synchronize()
-        assert torch.equal(w, want), trial
-        other = a[:512, :512] @ a[:512, :512]   # eager work between the replays
-        torch.cuda.synchronize()
-        del other
+    for capture_stream in (side, torch.cuda.Stream()):      # known to the library / never seen by it
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=capture_stream):
+            ops.lud(w)
+        for trial in range(3):
+            w.copy_(a)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(w, want), trial
+            other = a[:512, :512] @ a[:512, :512]   # eager work between the replays
+            torch.cuda.synchronize()
+            del other
+        del graph

@@ -170,3 +170,10 @@ def test_gpu_stencil_rejects_bad_arguments():
         ops.stencil_f3d(x, c, radius=4)
     with pytest.raises(LegoHipError):
         ops.stencil_f3d(torch.zeros(12, 12, 12, device="cuda"), c, radius=1)
+    # an `out` the kernel could not write through is refused before the launch
+    for bad in (torch.zeros(16, 16, 16), torch.zeros(16, 16, 16, device="cuda", dtype=torch.half),
+                torch.zeros(8, 16, 16, device="cuda"), torch.zeros(16, 16, 32, device="cuda")[:, :, ::2], x):
+        with pytest.raises(ValueError):
+            ops.stencil_f3d(x, c, radius=1, out=bad)
+        with pytest.raises(ValueError):
+            ops.stencil_laplacian(x, torch.zeros(2, device="cuda"), radius=1, out=bad)
