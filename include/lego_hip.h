@@ -97,9 +97,13 @@ int lego_hip_layernorm_bwd_bf16(const void* dy, const void* x, const void* w, co
 
 /* C = A * B, A is M x K, B is K x N, C is M x N, fp16 with fp32 accumulation.
  * Replaces matmul(a, b) (reference: triton_generated/matmul/matmul_NTA_NTB.py:129-145).
- * M and N multiples of 8 (one 16-byte chunk of fp16; the 256 x 256 tiles may be ragged at the
- * edges, which the reference kernel cannot be: no edge masks, matmul_sympy.py:196-203), K a
- * multiple of 64.  Shapes in whole tiles take a kernel without edge tests. */
+ * Any M, N, K (the reference keeps them symbolic and masks its tiles' edges, matmul_sympy.py:69-70,
+ * 196-203).  The MFMA kernels on 256 x 256 (or 128 x 128) tiles, ragged at the edges and with a masked
+ * last k-tile where need be, take every shape whose operand rows are whole 16-byte chunks on 16-byte
+ * aligned bases: N a multiple of 8, and K (operands as given) or M (A transposed) a multiple of 8 as
+ * well.  Any other shape or alignment (bases need only element alignment then) takes a kernel that
+ * moves one element per access, about a tenth as fast.  Shapes in whole tiles take a kernel without
+ * edge tests. */
 int lego_hip_gemm_f16(const void* a, const void* b, void* c, int M, int N, int K, void* stream);
 /* The same with the reference's fused epilogue (matmul(a, b, activation="leaky_relu"),
  * matmul_NTA_NTB.py:129-145): activation 0 = none, 1 = leaky_relu on the fp32 accumulator. */
@@ -117,7 +121,7 @@ int lego_hip_gemm_bf16_ex(const void* a, const void* b, void* c, int M, int N, i
 /* 8-bit floating-point operands, fp32 accumulation, fp16 result: the reference's fp8 path casts
  * both operands to float8_e5m2 and stores fp16 (matmul_sympy.py:346-364, 203).  format 0 = OCP
  * e4m3 (torch.float8_e4m3fn), 1 = OCP e5m2 (torch.float8_e5m2); a and b hold one byte per
- * element; M and N multiples of 16, K a multiple of 128. */
+ * element; shapes as for fp16, a 16-byte chunk being 16 elements and a k-tile 128. */
 int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                          int activation, int format, void* stream);
 
@@ -170,7 +174,9 @@ int lego_hip_nw_i32(const int* reference, int* matrix, int n, int penalty, void*
 
 /* groups independent GEMMs in one launch.  a, b, c are HOST arrays of `groups` device
  * pointers; sizes3 is a HOST array of groups*3 ints (M, N, K per problem).  At most 64
- * groups; every M, N a multiple of 8 and K a multiple of 64.  Replaces
+ * groups.  One launch when every N and K is a multiple of 8 and every base 16-byte aligned (any M;
+ * ragged tiles and last k-tiles are masked); otherwise one launch per problem, as lego_hip_gemm_f16
+ * would take it.  Replaces
  * lego_group_gemm_fn(group_A, group_B) (reference:
  * triton_generated/grouped_gemm/grouped_gemm.py:120-162), whose device-side tables are
  * passed here by value as kernel arguments, so no table is allocated or copied. */

@@ -91,6 +91,7 @@ def generate():
                                       trans_a=ta, trans_b=tb, dtype=dtype,
                                       with_grouped=dtype == "f16" and not (ta or tb))
                     units.append(gs)
+    units.append(gemm.emit_any())
     lb, mlb = layernorm_bwd.emit()
     units.append(lb)
     nwu, mnw = nw.emit()
@@ -149,6 +150,7 @@ def generate():
           "const int*, int, hipStream_t);",
           f"hipError_t lego_grouped_gemm_f16_t{GEMM_SMALL_TILE}x{GEMM_SMALL_TILE}_launch(const void* const*, "
           "const void* const*, void* const*, const int*, int, hipStream_t);",
+          "hipError_t lego_gemm_any_launch(const void*, const void*, void*, int, int, int, int, int, int, int, hipStream_t);",
           "hipError_t lego_grouped_gemm_f16_split_launch(const void* const*, const void* const*, void* const*, "
           "const int*, int, int, hipStream_t);",
           f"#define LEGO_GEMM_BM {mg['BM']}", f"#define LEGO_GEMM_BN {mg['BN']}", f"#define LEGO_GEMM_BK {mg['BK']}",

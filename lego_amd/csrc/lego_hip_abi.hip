@@ -288,13 +288,26 @@ struct GemmKernels {
 // keeps more of the 256 CUs busy than its higher LDS traffic per flop costs.
 constexpr long kSmallTileBelow = 129;
 
-int gemm_ex(const GemmKernels& k, const void* a, const void* b, void* c, int M, int N, int K,
+int gemm_ex(const GemmKernels& k, int element, const void* a, const void* b, void* c, int M, int N, int K,
             int trans_a, int trans_b, int activation, void* stream, int bk = LEGO_GEMM_BK, int chunk = 8)
 {
-  // M and N in whole 16-byte chunks (`chunk` elements), K in whole k-tiles; tiles may be ragged
-  if (!usable(a) || !usable(b) || !usable(c)) return kInvalid;
-  if (M <= 0 || N <= 0 || K <= 0 || M % chunk || N % chunk || K % bk) return kInvalid;
+  if (a == nullptr || b == nullptr || c == nullptr || M <= 0 || N <= 0 || K <= 0) return kInvalid;
   if (activation != 0 && activation != 1) return kInvalid;
+  // The tiled kernels move 16-byte chunks (`chunk` elements): bases 16-byte aligned and every operand row
+  // in whole chunks -- rows of C and of B as given run along N, rows of A as given and of a transposed B
+  // along K, rows of a transposed A along M.  Tiles may be ragged in M, N and K.  Everything else -- the
+  // reference keeps M, N, K symbolic (matmul_sympy.py:69-70) -- goes to the kernel that moves one element
+  // per access.
+  (void)bk;
+  const bool tiled = usable(a) && usable(b) && usable(c) && N % chunk == 0 &&
+                     (trans_a ? M % chunk == 0 : K % chunk == 0) && (!trans_b || K % chunk == 0);
+  if (!tiled) {
+    const uintptr_t in_mask = element <= 1 ? 1u : 0u;       // 2-byte or 1-byte operand elements; C is 2-byte
+    if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & in_mask) return kInvalid;
+    if (reinterpret_cast<uintptr_t>(c) & 1u) return kInvalid;
+    return ok_or(lego_gemm_any_launch(a, b, c, M, N, K, trans_a ? 1 : 0, trans_b ? 1 : 0, activation, element,
+                                      as_stream(stream)));
+  }
   const long tiles = static_cast<long>((M + LEGO_GEMM_BM - 1) / LEGO_GEMM_BM) * ((N + LEGO_GEMM_BN - 1) / LEGO_GEMM_BN);
   const gemm_launcher* by_layout = tiles < kSmallTileBelow && k.small[0] != nullptr ? k.small : k.big;
   return ok_or(by_layout[(trans_a ? 2 : 0) + (trans_b ? 1 : 0)](a, b, c, M, N, K, activation, as_stream(stream)));
@@ -315,14 +328,14 @@ int lego_hip_gemm_f16_ex(const void* a, const void* b, void* c, int M, int N, in
                          int activation, void* stream)
 {
   static const GemmKernels k = LEGO_GEMM_KERNELS(f16);
-  return gemm_ex(k, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
+  return gemm_ex(k, 0, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
 }
 
 int lego_hip_gemm_bf16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                           int activation, void* stream)
 {
   static const GemmKernels k = LEGO_GEMM_KERNELS(bf16);
-  return gemm_ex(k, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
+  return gemm_ex(k, 1, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
 }
 
 int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
@@ -331,8 +344,8 @@ int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, in
   static const GemmKernels e4m3 = LEGO_GEMM_KERNELS_BIG_ONLY(e4m3);
   static const GemmKernels e5m2 = LEGO_GEMM_KERNELS_BIG_ONLY(e5m2);
   if (format != 0 && format != 1) return kInvalid;
-  return gemm_ex(format == 0 ? e4m3 : e5m2, a, b, c, M, N, K, trans_a, trans_b, activation, stream,
-                 LEGO_GEMM_BK_8BIT, 16);
+  return gemm_ex(format == 0 ? e4m3 : e5m2, format == 0 ? 2 : 3, a, b, c, M, N, K, trans_a, trans_b, activation,
+                 stream, LEGO_GEMM_BK_8BIT, 16);
 }
 
 int lego_hip_gemm_f16_act(const void* a, const void* b, void* c, int M, int N, int K, int activation, void* stream)
@@ -460,7 +473,7 @@ GroupedPlan grouped_plan(const int* sizes3, int groups)
     const int m = sizes3[3 * g], n = sizes3[3 * g + 1];
     big[s] = static_cast<long>((m + 255) / 256) * ((n + 255) / 256);
     small[s] = static_cast<long>((m + 127) / 128) * ((n + 127) / 128);
-    depth[s] = sizes3[3 * g + 2] / LEGO_GEMM_BK;
+    depth[s] = (sizes3[3 * g + 2] + LEGO_GEMM_BK - 1) / LEGO_GEMM_BK;
     small_cost[s] = kSmallCost * (depth[s] + kTileOverhead);
     total += big[s];
   }
@@ -497,14 +510,33 @@ GroupedPlan grouped_plan(const int* sizes3, int groups)
   return plan;
 }
 
+// 0: every problem fits the tiled kernels (one launch); 2: the arguments are valid but some problem needs
+// the element-wise kernel (N or K not in whole 16-byte chunks, a base that is not 16-byte aligned);
+// kInvalid otherwise
 int grouped_check(const void* const* a, const void* const* b, void* const* c, const int* sizes3, int groups)
 {
   if (a == nullptr || b == nullptr || c == nullptr || sizes3 == nullptr) return kInvalid;
   if (groups <= 0 || groups > LEGO_GROUPED_MAX_GROUPS) return kInvalid;
+  int verdict = 0;
   for (int g = 0; g < groups; ++g) {
     const int m = sizes3[3 * g], n = sizes3[3 * g + 1], k = sizes3[3 * g + 2];
-    if (!usable(a[g]) || !usable(b[g]) || !usable(c[g])) return kInvalid;
-    if (m <= 0 || n <= 0 || k <= 0 || m % 8 || n % 8 || k % LEGO_GEMM_BK) return kInvalid;
+    if (a[g] == nullptr || b[g] == nullptr || c[g] == nullptr || m <= 0 || n <= 0 || k <= 0) return kInvalid;
+    if ((reinterpret_cast<uintptr_t>(a[g]) | reinterpret_cast<uintptr_t>(b[g]) | reinterpret_cast<uintptr_t>(c[g])) & 1u)
+      return kInvalid;
+    if (!usable(a[g]) || !usable(b[g]) || !usable(c[g]) || n % 8 || k % 8) verdict = 2;    // M may be anything
+  }
+  return verdict;
+}
+
+// A grouped call with a problem that the one-launch kernels do not take: one launch per problem on the
+// same stream, each through the plain GEMM's dispatch (the reference walks its problems in one kernel,
+// grouped_gemm.py:61-116, but takes whole tiles only).
+int grouped_one_by_one(const void* const* a, const void* const* b, void* const* c, const int* sizes3, int groups,
+                       void* stream)
+{
+  for (int g = 0; g < groups; ++g) {
+    const int err = lego_hip_gemm_f16_ex(a[g], b[g], c[g], sizes3[3 * g], sizes3[3 * g + 1], sizes3[3 * g + 2], 0, 0, 0, stream);
+    if (err != 0) return err;
   }
   return 0;
 }
@@ -513,7 +545,9 @@ int grouped_check(const void* const* a, const void* const* b, void* const* c, co
 int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* const* c,
                               const int* sizes3, int groups, void* stream)
 {
-  if (grouped_check(a, b, c, sizes3, groups) != 0) return kInvalid;
+  const int checked = grouped_check(a, b, c, sizes3, groups);
+  if (checked == 2) return grouped_one_by_one(a, b, c, sizes3, groups, stream);
+  if (checked != 0) return kInvalid;
   // One launch: on 256 x 256 tiles (one workgroup per CU), the last tiles of the launch order split
   // into halves when whole tiles would leave the last round mostly empty, or on 128 x 128 tiles (four
   // times as many workgroups of a quarter of the work, two per CU) when the big ones leave most CUs
@@ -541,7 +575,7 @@ int lego_hip_grouped_gemm_f16_plan(const int* sizes3, int groups, int* plan3)
 int lego_hip_grouped_gemm_f16_split(const void* const* a, const void* const* b, void* const* c,
                                     const int* sizes3, int groups, int split_tiles, void* stream)
 {
-  if (grouped_check(a, b, c, sizes3, groups) != 0) return kInvalid;
+  if (grouped_check(a, b, c, sizes3, groups) != 0) return kInvalid;     // tiled problems only
   if (split_tiles < 0)
     return ok_or(lego_grouped_gemm_f16_t128x128_launch(a, b, c, sizes3, groups, as_stream(stream)));
   return ok_or(lego_grouped_gemm_f16_split_launch(a, b, c, sizes3, groups, split_tiles, as_stream(stream)));

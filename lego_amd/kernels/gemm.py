@@ -251,8 +251,11 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
         # instruction) or its first column (the other kind: the same for every instruction)
         edge0, edge_step = chunk_walk(r_e if kmajor else col_e, n_iters)
         assert kmajor or edge_step == 0
+        # the first k-value (within the tile) of a lane's chunk: what a ragged last k-tile is masked by
+        kedge0, kedge_step = chunk_walk(EPC * ch_e if kmajor else kr_e, n_iters)
         return {f"{role}_src0": code(src0), f"{role}_src_step": code(step),
                 f"{role}_edge0": code(edge0), f"{role}_edge_step": code(edge_step),
+                f"{role}_kedge0": code(kedge0), f"{role}_kedge_step": code(kedge_step),
                 f"{role}_goff_base": code(full.subs({k: 0, row: 0, ch: 0, kr: 0})),
                 f"{role}_kstep": code(sp.simplify(full.subs(k, k + 1) - full)),
                 f"{role}_frag_code": frag}
@@ -327,3 +330,25 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
     if with_split:
         launchers.append(f"lego_grouped_gemm_f16{tag}_split_launch")
     return Emitted(f"gemm_{dtype}_{variant}{tag}.hip", text, launchers), meta
+
+
+def emit_any(bm=64, bn=64, bk=32):
+    """The kernel for shapes the tiled kernels do not take (any M, N, K and alignment): one element per
+    global access, operands staged k-major in LDS with zero fill past the edges."""
+    assert bm == 64 and bn == 64 and bk % 16 == 0 and 256 * 8 == bm * bk == bn * bk
+    M, N, K = size("M"), size("N"), size("K")
+    row, col, kk, sr, sk = (idx(n) for n in ("row", "col", "kk", "sr", "sk"))
+    rng = {row: (0, M), col: (0, N), kk: (0, K)}
+    flat = lambda lay, i, j: tidy(lay.TileBy([lay.dims()[0], lay.dims()[1]])[i, j], rng)  # noqa: E731
+    pitch = bk + 8        # 80-byte rows: eight-k reads of 32 consecutive rows cover every 16-byte bank group evenly
+    S = OrderBy(Row(bm, pitch)).TileBy([bm, pitch])
+    text = template("gemm_any.hip.j2").render(
+        banner=BANNER, BM=bm, BN=bn, BK=bk, PITCH=pitch,
+        a_row_layout="OrderBy(Row(M, K))[row, kk]", a_col_layout="OrderBy(Col(M, K))[row, kk]",
+        b_row_layout="OrderBy(Row(K, N))[kk, col]", b_col_layout="OrderBy(Col(K, N))[kk, col]",
+        c_layout="OrderBy(Row(M, N))[row, col]", s_layout=f"OrderBy(Row({bm}, {pitch}))[sr, sk]",
+        a_row=code(flat(OrderBy(Row(M, K)), row, kk)), a_col=code(flat(OrderBy(Col(M, K)), row, kk)),
+        b_row=code(flat(OrderBy(Row(K, N)), kk, col)), b_col=code(flat(OrderBy(Col(K, N)), kk, col)),
+        c_off=code(flat(OrderBy(Row(M, N)), row, col)),
+        s_off=code(tidy(S[sr, sk], {sr: (0, bm), sk: (0, pitch)})))
+    return Emitted("gemm_any.hip", text, ["lego_gemm_any_launch"])

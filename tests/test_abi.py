@@ -42,7 +42,9 @@ def test_argument_validation_needs_no_gpu():
     assert lib.lego_hip_softmax_f32(ctypes.c_void_p(16), ctypes.c_void_p(4096), 0, 64, None) == 1
     assert lib.lego_hip_softmax_f16_wpr(ctypes.c_void_p(16), ctypes.c_void_p(4096), 4, 32776, 16, None) == 1
     assert lib.lego_hip_softmax_f16_wpr(ctypes.c_void_p(16), ctypes.c_void_p(4096), 4, 1024, 3, None) == 1      # no such team
-    assert lib.lego_hip_gemm_f16(ctypes.c_void_p(16), ctypes.c_void_p(32), ctypes.c_void_p(64), 256, 100, 64, None) == 1
+    assert lib.lego_hip_gemm_f16(ctypes.c_void_p(16), ctypes.c_void_p(32), ctypes.c_void_p(64), 256, 0, 64, None) == 1
+    assert lib.lego_hip_gemm_f16(ctypes.c_void_p(17), ctypes.c_void_p(32), ctypes.c_void_p(64), 256, 100, 64, None) == 1
+    assert lib.lego_hip_gemm_f16_ex(ctypes.c_void_p(16), ctypes.c_void_p(32), ctypes.c_void_p(64), 8, 8, 64, 0, 0, 2, None) == 1
     assert lib.lego_hip_grouped_gemm_f16(None, None, None, None, 1, None) == 1
     with pytest.raises(runtime.LegoHipError):
         runtime.call("lego_hip_transpose_f32", None, None, 64, 64, None)

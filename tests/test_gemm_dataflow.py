@@ -159,3 +159,43 @@ def test_ragged_edges_skip_exactly_what_lies_outside(variant, tile):
                             assert 0 <= r_ < rem and 0 <= k_ < bk, (role, rem, wave, lane, it)
                             covered.add((r_, k_))
             assert covered == {(r, k) for r in range(rem) for k in range(bk)}, (role, rem)
+
+
+@pytest.mark.parametrize("dtype,bk", [("f16", 64), ("e5m2", 128)])
+@pytest.mark.parametrize("variant", ["nn", "tt"])
+def test_last_k_tile_zeroes_exactly_what_lies_past_k(dtype, bk, variant):
+    """The EDGE instantiation guards every slot of the last k-tile with ``k0 + X*step >= klim``: such a slot
+    is written as zeros, the others are fetched.  For every ``klim`` in whole chunks, replay the guards
+    over all slots: a slot is zeroed exactly when the chunk that the layout puts there starts at or past
+    ``klim`` (chunks never straddle it), so the tile ends up holding the operand's k-values below
+    ``klim`` and zeros above."""
+    ta, tb = variant[0] == "t", variant[1] == "t"
+    tile = 256
+    unit, _ = gemm.emit(bm=tile, bn=tile, bk=bk, trans_a=ta, trans_b=tb, with_grouped=False, dtype=dtype)
+    text = unit.text
+    esize = 2 if dtype == "f16" else 1
+    epc = 16 // esize
+    K = 2 * bk
+    sizes = dict(M=512, N=512, K=K)
+    k0s = _grab(text, r"const unsigned a_k0 = (.*), b_k0 = .*;"), _grab(text, r"const unsigned a_k0 = .*, b_k0 = (.*);")
+    for role, rows_total, kmajor, k0_text in (("a", 512, not ta, k0s[0]), ("b", 512, tb, k0s[1])):
+        src0 = _grab(text, r"const unsigned %s_src0 = \d \* \((.*)\);" % role)
+        step = _grab(text, r"%s_src_step = \d \* \((.*?)\)[,;]" % role)
+        kstep = int(_grab(text, r"%s_k0 \+ \(.*?\) \* \((\d+)\) >= klim_nx" % role))
+        iters = tile * bk // epc // 256
+        for klim in range(epc, bk + 1, epc):
+            zeroed, fetched = set(), set()
+            for wave in range(4):
+                for lane in range(64):
+                    base = _c_eval(src0, dict(sizes, wave=wave, lane=lane))
+                    k0 = _c_eval(k0_text, dict(wave=wave, lane=lane))
+                    for it in range(iters):
+                        off = base + it * _c_eval(step, sizes)
+                        r_, k_ = divmod(off, K) if kmajor else divmod(off, rows_total)[::-1]
+                        assert k_ == k0 + it * kstep, (role, wave, lane, it)      # the guard sees the chunk's own k
+                        (zeroed if k0 + it * kstep >= klim else fetched).add((r_, k_))
+            if kmajor:
+                assert fetched == {(r, k) for r in range(tile) for k in range(0, klim, epc)}
+            else:
+                assert fetched == {(r, k) for r in range(0, tile, epc) for k in range(klim)}
+            assert len(zeroed) + len(fetched) == tile * bk // epc

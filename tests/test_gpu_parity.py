@@ -550,6 +550,77 @@ def test_grouped_gemm_many_tiles_unsorted_depths(ops):
         assert _rel_err(c.cpu(), w) <= 1e-2
 
 
+# ---- GEMM shapes outside the tiled kernels: any M, N, K and alignment (matmul_sympy.py:69-70, 196-203) ----
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float8_e5m2, torch.float8_e4m3fn])
+@pytest.mark.parametrize("M,N,K", [(1001, 263, 100), (1, 1, 1), (65, 64, 33), (1024, 512, 200), (1000, 264, 72),
+                                   (1001, 264, 200), (1008, 528, 208), (300, 4104, 8), (2056, 2056, 1000)])
+def test_gemm_any_shape_all_layouts(ops, dtype, M, N, K):
+    """M, N, K of any size, the four operand layouts, with and without the fused leaky_relu.  Shapes whose
+    operand rows are whole 16-byte chunks take the tiled kernels with ragged tiles and a masked last
+    k-tile ((1024, 512, 200), (1000, 264, 72), (1008, 528, 208) for every element type, (1001, 264, 200)
+    where A is stored row-major, K = 8 is a single, mostly masked k-tile); the others the kernel that
+    moves one element per access."""
+    print(f"gemm any shape {dtype} {M}x{N}x{K}", flush=True)
+    g = _gen(41)
+    a = (torch.randn(M, K, generator=g) / math.sqrt(K)).half().to(dtype)
+    b = (torch.randn(K, N, generator=g) / math.sqrt(K)).half().to(dtype)
+    want = a.float() @ b.float()
+    out_dtype = torch.float16 if dtype in (torch.float8_e5m2, torch.float8_e4m3fn) else dtype
+    tol = 2.0 ** -8 if out_dtype == torch.bfloat16 else 2.0 ** -10           # the store's rounding + accumulation order
+    for ta in (False, True):
+        for tb in (False, True):
+            ad = a.t().contiguous().cuda().t() if ta else a.cuda()
+            bd = b.t().contiguous().cuda().t() if tb else b.cuda()
+            got = ops.matmul(ad, bd)
+            assert got.dtype == out_dtype and got.shape == (M, N)
+            assert ((got.cpu().float() - want).abs() <= tol * want.abs() + 1e-3).all(), (ta, tb)
+            act = ops.matmul(ad, bd, activation="leaky_relu").cpu().float()
+            want_act = torch.where(want >= 0, want, 0.01 * want)
+            assert ((act - want_act).abs() <= tol * want_act.abs() + 1e-3).all(), (ta, tb)
+
+
+def test_gemm_any_shape_is_exact_on_small_integers(ops):
+    """Integer operands with exactly representable sums: every element of every ragged tile, bit for bit."""
+    print("gemm any shape, integers", flush=True)
+    g = _gen(42)
+    M, N, K = 193, 131, 77
+    a = torch.randint(-3, 4, (M, K), generator=g).half()
+    b = torch.randint(-3, 4, (K, N), generator=g).half()
+    want = (a.double() @ b.double()).half()
+    for ta in (False, True):
+        for tb in (False, True):
+            ad = a.t().contiguous().cuda().t() if ta else a.cuda()
+            bd = b.t().contiguous().cuda().t() if tb else b.cuda()
+            assert torch.equal(ops.matmul(ad, bd).cpu(), want), (ta, tb)
+
+
+def test_gemm_operands_at_any_element_alignment(ops):
+    """Whole-tile shapes whose bases are not 16-byte aligned (views that start one element into a buffer)."""
+    print("gemm misaligned bases", flush=True)
+    g = _gen(43)
+    M, N, K = 256, 256, 128
+    a = (torch.randn(M * K + 1, generator=g) / math.sqrt(K)).half().cuda()[1:].view(M, K)
+    b = (torch.randn(K * N + 3, generator=g) / math.sqrt(K)).half().cuda()[3:].view(K, N)
+    assert a.data_ptr() % 16 and b.data_ptr() % 16
+    got = ops.matmul(a, b).cpu()
+    assert _rel_err(got, ok.gemm(a.cpu(), b.cpu())) <= 1e-2
+
+
+def test_grouped_gemm_with_odd_problems(ops):
+    """A grouped call with problems outside the tiled kernels falls back to one launch per problem."""
+    print("grouped gemm, odd problems", flush=True)
+    g = _gen(44)
+    shapes = [(512, 256, 128), (1001, 263, 100), (64, 72, 200), (7, 5, 3)]
+    A = [(torch.randn(m, k, generator=g) / math.sqrt(k)).half() for m, n, k in shapes]
+    B = [(torch.randn(k, n, generator=g) / math.sqrt(k)).half() for m, n, k in shapes]
+    want = ok.grouped_gemm(A, B)
+    got = ops.lego_group_gemm_fn([a.cuda() for a in A], [b.cuda() for b in B])
+    for c, w in zip(got, want):
+        assert c.shape == w.shape
+        assert ((c.cpu().float() - w.float()).abs() <= 2.0 ** -9 * w.float().abs() + 1e-3).all()
+
+
 def _grouped_call(entry, A, B, *extra):
     """Call a grouped entry point through the C ABI on device tensors; returns the results."""
     import ctypes
@@ -711,10 +782,12 @@ def test_gemm_offsets_beyond_32_bits(ops):
         assert _rel_err(c[rows].cpu(), ok.gemm(a[rows].cpu(), b.cpu())) <= 1e-2
 
 
-def test_gemm_rejects_bad_shapes(ops):
-    from lego_amd.runtime import LegoHipError
-    with pytest.raises(LegoHipError):
+def test_gemm_rejects_bad_arguments(ops):
+    with pytest.raises(ValueError):          # inner dimensions differ
         ops.matmul(torch.zeros(100, 64, device="cuda", dtype=torch.half),
+                   torch.zeros(72, 256, device="cuda", dtype=torch.half))
+    with pytest.raises(ValueError):          # neither the operand nor its transpose is contiguous
+        ops.matmul(torch.zeros(100, 128, device="cuda", dtype=torch.half)[:, ::2],
                    torch.zeros(64, 256, device="cuda", dtype=torch.half))
     with pytest.raises(NotImplementedError):
         ops.matmul(torch.zeros(256, 64, device="cuda", dtype=torch.half),
