@@ -118,6 +118,10 @@ int lego_hip_gemm_f16_ex(const void* a, const void* b, void* c, int M, int N, in
  * here the result has the operands' type. */
 int lego_hip_gemm_bf16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                           int activation, void* stream);
+/* bfloat16 operands, fp16 result: what the reference's matmul returns for bfloat16 tensors (it stores
+ * `accumulator.to(tl.float16)` into a float16 tensor whatever its operands' type, matmul_sympy.py:136, 203). */
+int lego_hip_gemm_bf16_f16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
+                              int activation, void* stream);
 /* 8-bit floating-point operands, fp32 accumulation, fp16 result: the reference's fp8 path casts
  * both operands to float8_e5m2 and stores fp16 (matmul_sympy.py:346-364, 203).  format 0 = OCP
  * e4m3 (torch.float8_e4m3fn), 1 = OCP e5m2 (torch.float8_e5m2); a and b hold one byte per

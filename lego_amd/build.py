@@ -51,9 +51,9 @@ ROWWISE_WIDE_TEAM_ABOVE_N, ROWWISE_WIDE_TEAM_FROM_M = 6144, 4096
 ROWWISE_MAX_N = rowwise.MAX_N
 GEMM = dict(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8)
 GEMM_SMALL_TILE = 128
-GEMM_SMALL_DTYPES = ("f16", "bf16")     # a 128-byte row of 8-bit elements is too short for their [k][n] rotation
-GEMM_DTYPES = ("f16", "bf16", "e4m3", "e5m2")
-GEMM_BK = {"f16": 64, "bf16": 64, "e4m3": 128, "e5m2": 128}   # 128 bytes of k per operand row in every case
+GEMM_SMALL_DTYPES = ("f16", "bf16", "bf16h")     # a 128-byte row of 8-bit elements is too short for their [k][n] rotation
+GEMM_DTYPES = ("f16", "bf16", "bf16h", "e4m3", "e5m2")     # bf16h: bfloat16 operands, fp16 result
+GEMM_BK = {"f16": 64, "bf16": 64, "bf16h": 64, "e4m3": 128, "e5m2": 128}   # 128 bytes of k per operand row in every case
 
 
 def generate():

@@ -302,7 +302,7 @@ int gemm_ex(const GemmKernels& k, int element, const void* a, const void* b, voi
   const bool tiled = usable(a) && usable(b) && usable(c) && N % chunk == 0 &&
                      (trans_a ? M % chunk == 0 : K % chunk == 0) && (!trans_b || K % chunk == 0);
   if (!tiled) {
-    const uintptr_t in_mask = element <= 1 ? 1u : 0u;       // 2-byte or 1-byte operand elements; C is 2-byte
+    const uintptr_t in_mask = element <= 1 || element == 4 ? 1u : 0u;       // 2-byte or 1-byte operand elements; C is 2-byte
     if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & in_mask) return kInvalid;
     if (reinterpret_cast<uintptr_t>(c) & 1u) return kInvalid;
     return ok_or(lego_gemm_any_launch(a, b, c, M, N, K, trans_a ? 1 : 0, trans_b ? 1 : 0, activation, element,
@@ -336,6 +336,13 @@ int lego_hip_gemm_bf16_ex(const void* a, const void* b, void* c, int M, int N, i
 {
   static const GemmKernels k = LEGO_GEMM_KERNELS(bf16);
   return gemm_ex(k, 1, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
+}
+
+int lego_hip_gemm_bf16_f16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
+                              int activation, void* stream)
+{
+  static const GemmKernels k = LEGO_GEMM_KERNELS(bf16h);
+  return gemm_ex(k, 4, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
 }
 
 int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,

@@ -108,7 +108,10 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
     """Everything the templates need for one tile shape."""
     # element type, bytes per element, k-depth of one MFMA, result type; the 8-bit types are the
     # OCP formats of v_mfma_f32_32x32x64_f8f6f4 (format code 0 = e4m3, 1 = e5m2)
+    # "bf16h": bfloat16 operands with the fp16 result that the reference's matmul stores whatever its
+    # operands' 16-bit type (matmul_sympy.py:129-145, 203)
     elt, esize, mfma_k, out_elt = {"f16": ("_Float16", 2, 16, "_Float16"), "bf16": ("__bf16", 2, 16, "__bf16"),
+                                   "bf16h": ("__bf16", 2, 16, "_Float16"),
                                    "e4m3": ("unsigned char", 1, 64, "_Float16"),
                                    "e5m2": ("unsigned char", 1, 64, "_Float16")}[dtype]
     EPC = 16 // esize                      # elements per 16-byte chunk
@@ -266,7 +269,7 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
 
     params = dict(
         banner=BANNER, elt=elt, out_elt=out_elt, ESIZE=esize, EPC=EPC, MFMA_K=mfma_k, NPH=NPH,
-        FMT={"e4m3": 0, "e5m2": 1}.get(dtype, 0), dt=dtype, BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
+        FMT={"e4m3": 0, "e5m2": 1}.get(dtype, 0), dt=dtype, mfma_dt={"bf16h": "bf16"}.get(dtype, dtype), BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
         WM=WM, WN=WN, TM=TM, TN=TN, A_ITERS=A_ITERS, B_ITERS=B_ITERS, DMA_LAST=DMA_LAST,
         load_slots=load_slots, dma_last=dma_last, dma_first=dma_first, dma_none=none, XCDS=XCDS, MAX_GROUPS=MAX_GROUPS,
         pid_layout="OrderBy(Col(max(npm//GM,1),1), Col(min(npm,GM),npn)).TileBy([npm,npn]).inv(pid)",

@@ -174,10 +174,11 @@ def _operand(t, name):
     raise ValueError(f"{name} must be contiguous or the transpose of a contiguous tensor")
 
 
-def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "") -> torch.Tensor:
-    """``act(a @ b)`` for fp16 (or bf16) operands, each row-major or column-major (a ``.T``
-    view), fp32 accumulation, row-major result of the operands' type.  float8_e5m2 (the
-    reference's fp8 path, matmul_sympy.py:346-364) and float8_e4m3fn operands give an fp16 result."""
+def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "", out_dtype=torch.float16) -> torch.Tensor:
+    """``act(a @ b)`` for fp16, bf16 or 8-bit floating-point operands of any shape, each row-major or
+    column-major (a ``.T`` view), fp32 accumulation, row-major fp16 result: the reference's ``matmul``
+    allocates a float16 result whatever its operands' type (matmul_sympy.py:129-145, its fp8 path
+    :346-364).  ``out_dtype=torch.bfloat16`` with bfloat16 operands keeps their type instead."""
     if activation not in ("", "leaky_relu"):
         raise NotImplementedError(f"activation {activation!r} is not generated by this build")
     a_store, ta = _operand(a, "a")
@@ -193,9 +194,11 @@ def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "") -> torch.Tens
         runtime.call("lego_hip_gemm_fp8_ex", _ptr(a_store), _ptr(b_store), _ptr(c), M, N, K, ta, tb,
                      1 if activation else 0, _FP8_FORMAT[a.dtype], _stream())
         return c
-    c = torch.empty((M, N), device=a.device, dtype=a.dtype)
-    runtime.call(_GEMM_ENTRY[a.dtype], _ptr(a_store), _ptr(b_store), _ptr(c), M, N, K, ta, tb,
-                 1 if activation else 0, _stream())
+    if out_dtype not in (torch.float16, a.dtype):
+        raise ValueError("out_dtype must be float16 or the operands' type")
+    entry = "lego_hip_gemm_bf16_f16_ex" if (a.dtype, out_dtype) == (torch.bfloat16, torch.float16) else _GEMM_ENTRY[a.dtype]
+    c = torch.empty((M, N), device=a.device, dtype=out_dtype)
+    runtime.call(entry, _ptr(a_store), _ptr(b_store), _ptr(c), M, N, K, ta, tb, 1 if activation else 0, _stream())
     return c
 
 

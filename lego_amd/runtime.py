@@ -35,6 +35,8 @@ SIGNATURES = {
                              _c_void_p],
     "lego_hip_gemm_bf16_ex": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                              _c_void_p],
+    "lego_hip_gemm_bf16_f16_ex": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                  _c_void_p],
     "lego_hip_gemm_fp8_ex": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                              _c_int, _c_void_p],
     "lego_hip_stencil_f3d_f32": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],

@@ -566,15 +566,18 @@ def test_gemm_any_shape_all_layouts(ops, dtype, M, N, K):
     a = (torch.randn(M, K, generator=g) / math.sqrt(K)).half().to(dtype)
     b = (torch.randn(K, N, generator=g) / math.sqrt(K)).half().to(dtype)
     want = a.float() @ b.float()
-    out_dtype = torch.float16 if dtype in (torch.float8_e5m2, torch.float8_e4m3fn) else dtype
-    tol = 2.0 ** -8 if out_dtype == torch.bfloat16 else 2.0 ** -10           # the store's rounding + accumulation order
+    tol = 2.0 ** -10           # the fp16 store's rounding + accumulation order
     for ta in (False, True):
         for tb in (False, True):
             ad = a.t().contiguous().cuda().t() if ta else a.cuda()
             bd = b.t().contiguous().cuda().t() if tb else b.cuda()
             got = ops.matmul(ad, bd)
-            assert got.dtype == out_dtype and got.shape == (M, N)
+            assert got.dtype == torch.float16 and got.shape == (M, N)      # the reference stores fp16 whatever the operands
             assert ((got.cpu().float() - want).abs() <= tol * want.abs() + 1e-3).all(), (ta, tb)
+            if dtype == torch.bfloat16:
+                own = ops.matmul(ad, bd, out_dtype=torch.bfloat16)
+                assert own.dtype == torch.bfloat16
+                assert ((own.cpu().float() - want).abs() <= 2.0 ** -8 * want.abs() + 1e-3).all(), (ta, tb)
             act = ops.matmul(ad, bd, activation="leaky_relu").cpu().float()
             want_act = torch.where(want >= 0, want, 0.01 * want)
             assert ((act - want_act).abs() <= tol * want_act.abs() + 1e-3).all(), (ta, tb)
@@ -836,11 +839,16 @@ def test_gemm_bf16_matches_oracle(ops, ta, tb):
     want = ok.gemm(a, b)
     ad = a.t().contiguous().cuda().t() if ta else a.cuda()
     bd = b.t().contiguous().cuda().t() if tb else b.cuda()
-    got = ops.matmul(ad, bd)
+    got = ops.matmul(ad, bd, out_dtype=torch.bfloat16)
     assert got.dtype == torch.bfloat16
     assert _rel_err(got.cpu(), want) <= 1e-2
     # round-to-nearest-even of the fp32 accumulator: at most one bf16 spacing from the oracle
     assert (got.cpu().float() - want.float()).abs().max().item() <= 2.0 ** -7
+    # the default is the reference's: an fp16 result whatever the operands' 16-bit type (matmul_sympy.py:136)
+    half = ops.matmul(ad, bd)
+    assert half.dtype == torch.float16
+    exact = a.float() @ b.float()
+    assert ((half.cpu().float() - exact).abs() <= 2.0 ** -10 * exact.abs() + 1e-4).all()
 
 
 def test_gemm_bf16_integer_exact(ops):
