@@ -56,8 +56,8 @@ GEMM_DTYPES = ("f16", "bf16", "bf16h", "e4m3", "e5m2")     # bf16h: bfloat16 ope
 GEMM_BK = {"f16": 64, "bf16": 64, "bf16h": 64, "e4m3": 128, "e5m2": 128}   # 128 bytes of k per operand row in every case
 
 
-def generate():
-    """Write every generated source; returns the list of .hip paths to compile."""
+def collect():
+    """Run every generator: ``(units, text of launchers.h)``, nothing written."""
     units = []
     tmeta = {}
     for dtype, configs in TRANSPOSE.items():
@@ -161,12 +161,21 @@ def generate():
           "hipError_t lego_stencil_f32_launch(const float*, float*, const float*, int, int, int, int, hipStream_t);",
           f"#define LEGO_STENCIL_BRICK {mst['B']}", f"#define LEGO_STENCIL_MAX_RADIUS {mst['MAX_RADIUS']}", "",
           "hipError_t lego_lud_f32_launch(float*, int, hipStream_t);", "hipError_t lego_lud_f32_plan(int, int*, int, int*);", f"#define LEGO_LUD_BLOCK {mlu['B']}", ""]
+    return units, "\n".join(h)
+
+
+def generate():
+    """Write every generated source; returns the list of .hip paths to compile."""
+    units, text = collect()
     GENERATED.mkdir(parents=True, exist_ok=True)
     header = GENERATED / "launchers.h"
-    text = "\n".join(h)
     if not header.exists() or header.read_text() != text:
         header.write_text(text)
-    return [u.write() for u in units]
+    paths = [u.write() for u in units]
+    # sources of translation units that are no longer generated would still be found by a glob: remove them
+    for stale in set(GENERATED.glob("*.hip")) - set(paths):
+        stale.unlink()
+    return paths
 
 
 def _compile(src: Path, incremental: bool = False) -> Path:

@@ -93,3 +93,29 @@ def transpose_smem(n, dtype="f32"):
                 j, i = pargs
                 TB[wby, wbx, i, j, rty, rtx] = TS[j, i, wty, wtx]
     return module
+
+
+def row_sums(rows, cols, dtype="f32"):
+    """``out[r] = sum_c A[r][c]``: a loop that carries its running sum, the builder's counterpart of the
+    reference's ``affine.for ... iter_args`` (lego/lego_mlir.py:85-108).  One lane per row, 64 lanes per
+    workgroup; no reference program uses a carried value, this one exists to exercise that path."""
+    assert rows % 64 == 0
+    grid, block = (rows // 64, 1, 1), (64, 1, 1)
+
+    @printer.generate_hip(name=f"lego_dsl_row_sums_{dtype}_{rows}x{cols}")
+    def module():
+        TA = HipTensor(OrderBy(Row(rows, cols)).TileBy([rows // 64, 1], [64, cols]), dtype)
+        TS = HipTensor(OrderBy(Row(rows)).TileBy([rows // 64], [64]), dtype)
+
+        @printer.generate_gpu_kernel([TA], [TS], grid, block)
+        def kernel(_):
+            bX = printer.get_block_linear_index()
+            tX = printer.get_thread_linear_index()
+
+            @printer.generate_loop(OrderBy(Row(cols)).TileBy([cols]), iter_args=[0.0])
+            def total(pargs, _, carried):
+                (c,) = pargs
+                return carried[0] + TA[bX, 0, tX, c]
+            (acc,) = total()
+            TS[bX, tX] = acc
+    return module

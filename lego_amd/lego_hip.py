@@ -165,6 +165,29 @@ class HipValue:
     def __str__(self):
         return self.name
 
+    # arithmetic on temporaries prints as C++ expressions (the MLIR builder's arith ops on SSA values)
+    def _binary(self, op, other, swap=False):
+        a, b = (other, self) if swap else (self, other)
+        return HipValue(f"({a} {op} {b})", self.ctype)
+
+    def __add__(self, other):
+        return self._binary("+", other)
+
+    def __radd__(self, other):
+        return self._binary("+", other, swap=True)
+
+    def __sub__(self, other):
+        return self._binary("-", other)
+
+    def __rsub__(self, other):
+        return self._binary("-", other, swap=True)
+
+    def __mul__(self, other):
+        return self._binary("*", other)
+
+    def __rmul__(self, other):
+        return self._binary("*", other, swap=True)
+
 
 class _Emitter:
     def __init__(self):
@@ -257,21 +280,54 @@ class HipKernelBuilder:
     def generate_loop(self, l: GroupBy, step=1, iter_args=()):
         """``for`` over ``prod(l.dims())`` steps; the body receives the logical index
         ``l.inv(i)`` and the flat counter (lego/lego_mlir.py:85-108).  The loop is emitted
-        with ``#pragma unroll`` because its trip count is a generation-time constant."""
-        if iter_args:
-            raise NotImplementedError("loop-carried values are not used by any HIP generator")
+        with ``#pragma unroll`` because its trip count is a generation-time constant.
 
-        def decorator(body):
+        With ``iter_args`` (initial values: temporaries or literals) the loop carries values, as the
+        reference's ``affine.for ... iter_args``: each becomes a named C++ temporary, the body
+        receives them as a third argument and returns their next values, and -- as in the
+        reference, where the decorated name is then bound to a function -- the decorator returns a
+        callable that emits the loop when called and returns the carried temporaries as they stand
+        after the last step.  ``ctype`` of a carried value: that of its initial temporary, ``float``
+        for a literal."""
+        carried = tuple(iter_args)
+
+        def emit_loop(body):
             em = self._em
+            carries = []
+            for init in carried:
+                ctype = init.ctype if isinstance(init, HipValue) else ("float" if isinstance(init, float) else "unsigned")
+                carry = HipValue(em.fresh("carry"), ctype)
+                em.emit(f"{ctype} {carry} = {init};")
+                carries.append(carry)
             var = em.fresh("it")
             trip = self._code.doprint(sp.sympify(product(l.dims())))
             em.emit("#pragma unroll")
             em.emit(f"for (unsigned {var} = 0; {var} < {trip}; {var} += {int(step)}) {{")
             em.depth += 1
             idx = sp.Symbol(var, integer=True, nonnegative=True)
-            body(l.inv(idx), idx)
+            if carries:
+                nxt = body(l.inv(idx), idx, tuple(carries))
+                nxt = tuple(nxt) if isinstance(nxt, (tuple, list)) else (nxt,)
+                if len(nxt) != len(carries):
+                    raise ValueError("the loop body must return one value per iter_arg")
+                # all next values are formed before any carried temporary changes, as a yield does
+                tmps = []
+                for carry, value in zip(carries, nxt):
+                    tmp = em.fresh("next")
+                    em.emit(f"const {carry.ctype} {tmp} = {value};")
+                    tmps.append(tmp)
+                for carry, tmp in zip(carries, tmps):
+                    em.emit(f"{carry} = {tmp};")
+            else:
+                body(l.inv(idx), idx)
             em.depth -= 1
             em.emit("}")
+            return tuple(carries)
+
+        def decorator(body):
+            if carried:
+                return lambda: emit_loop(body)
+            emit_loop(body)
         return decorator
 
     def get_block_linear_index(self):

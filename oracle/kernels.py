@@ -96,8 +96,10 @@ def grouped_pid(pid, num_pid_m, num_pid_n, group_m):
 
 
 def needleman_wunsch(reference, penalty):
-    """Rodinia's Needleman-Wunsch recurrence (benchmarks/cuda/nw/needle.cu:289-310, the reference's
-    own CPU check): borders ``-i*penalty``, then
+    """Rodinia's Needleman-Wunsch recurrence as the reference's kernels state it per cell
+    (benchmarks/cuda/nw/needle_kernel_temp.cu:70-258: ``maximum(nw + ref, w - penalty, n - penalty)`` over
+    the anti-diagonals of a tile; host loop and borders benchmarks/cuda/nw/needle.cu:165-260): borders
+    ``-i*penalty``, then
     ``m[i][j] = max(m[i-1][j-1] + ref[i][j], m[i][j-1] - penalty, m[i-1][j] - penalty)``,
     evaluated one anti-diagonal at a time with numpy.  ``reference`` is ``(n+1) x (n+1)`` int32."""
     ref = np.asarray(reference, dtype=np.int64)
@@ -123,46 +125,35 @@ def bricks_order(n, b=8):
 
 
 def stencil_f3d(x, c, radius):
-    """The dense stencil of benchmarks/cuda/bricks/main_tmp.cu:24-66 on a row-major ``n^3`` float32
-    array, in float64: the centre is weighted once on its own and once more inside the window
-    sum, boundary points are zero."""
+    """The dense stencil of benchmarks/cuda/bricks/main_tmp.cu:24-66 on a row-major float32 array (a cube,
+    or any box: a slab of a cube gives the cube's values on its inner planes), in float64: the centre
+    is weighted once on its own and once more inside the window sum, boundary points are zero."""
     x = np.asarray(x, dtype=np.float64)
     c = np.asarray(c, dtype=np.float64)
-    n, r = x.shape[0], radius
+    (n0, n1, n2), r = x.shape, radius
     out = np.zeros_like(x)
-    core = (slice(r, n - r),) * 3
+    core = (slice(r, n0 - r), slice(r, n1 - r), slice(r, n2 - r))
     acc = x[core] * c[r, r, r]
     for di in range(-r, r + 1):
         for dj in range(-r, r + 1):
             for dk in range(-r, r + 1):
-                acc = acc + x[r + di:n - r + di, r + dj:n - r + dj, r + dk:n - r + dk] * c[di + r, dj + r, dk + r]
+                acc = acc + x[r + di:n0 - r + di, r + dj:n1 - r + dj, r + dk:n2 - r + dk] * c[di + r, dj + r, dk + r]
     out[core] = acc
     return out
 
 
 def stencil_laplacian(x, c, radius):
-    """The star stencil of benchmarks/cuda/bricks-laplace/main_tmp.cu:24-57, in float64."""
+    """The star stencil of benchmarks/cuda/bricks-laplace/main_tmp.cu:24-57, in float64 (cube or box)."""
     x = np.asarray(x, dtype=np.float64)
     c = np.asarray(c, dtype=np.float64)
-    n, r = x.shape[0], radius
+    (n0, n1, n2), r = x.shape, radius
     out = np.zeros_like(x)
-    core = (slice(r, n - r),) * 3
+    core = (slice(r, n0 - r), slice(r, n1 - r), slice(r, n2 - r))
+    i, j, k = core
+    sh = lambda s_, a: slice(s_.start + a, s_.stop + a)      # noqa: E731
     acc = x[core] * c[0]
     for a in range(1, r + 1):
-        acc = acc + c[a] * (x[r + a:n - r + a, r:n - r, r:n - r] + x[r - a:n - r - a, r:n - r, r:n - r]
-                            + x[r:n - r, r + a:n - r + a, r:n - r] + x[r:n - r, r - a:n - r - a, r:n - r]
-                            + x[r:n - r, r:n - r, r + a:n - r + a] + x[r:n - r, r:n - r, r - a:n - r - a])
+        acc = acc + c[a] * (x[sh(i, a), j, k] + x[sh(i, -a), j, k] + x[i, sh(j, a), k] + x[i, sh(j, -a), k]
+                            + x[i, j, sh(k, a)] + x[i, j, sh(k, -a)])
     out[core] = acc
     return out
-
-
-def lud(a):
-    """LU decomposition without pivoting (Doolittle, unit lower triangle), what Rodinia's
-    ``lud_base`` computes (the reference's CPU check, benchmarks/cuda/lud/lud.cu with common.c), in
-    float64: returns one matrix with L below the diagonal and U on and above it."""
-    m = np.array(a, dtype=np.float64)
-    n = m.shape[0]
-    for k in range(n - 1):
-        m[k + 1:, k] /= m[k, k]
-        m[k + 1:, k + 1:] -= np.outer(m[k + 1:, k], m[k, k + 1:])
-    return m

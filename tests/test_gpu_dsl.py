@@ -19,3 +19,15 @@ def test_dsl_transpose(kind, n):
     mod.launch(mod.launchers[0], x, y, stream=torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     assert torch.equal(y, x.t())
+
+
+def test_dsl_loop_carried_row_sums():
+    print("dsl row sums", flush=True)
+    from lego_amd.kernels.dsl_transpose import row_sums
+    mod = row_sums(256, 96)
+    assert mod.so_path.exists(), "builder-DSL modules are compiled by __graft_entry__.build()"
+    x = torch.randint(-8, 9, (256, 96), generator=torch.Generator().manual_seed(0)).float().cuda()   # exact sums
+    y = torch.empty(256, device="cuda")
+    mod.launch(mod.launchers[0], x, y, stream=torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(y, x.sum(1))

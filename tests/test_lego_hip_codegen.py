@@ -112,3 +112,46 @@ def test_mod_by_a_power_is_parenthesised():
             for nv in (2, 3, 5):
                 assert eval(text.replace("/", "//"), {}, {"w": wv, "n": nv}) == (wv % (nv * nv)) // nv
         assert printer.doprint(sp.Mod(n**2, 7)) == "(n*n) % 7"
+
+
+def test_loops_carry_values():
+    """``generate_loop(iter_args=...)``: carried values become named temporaries, the body's return
+    values are assigned after all of them are formed, and the decorated name is a callable that
+    returns the temporaries (the reference binds it to a function as well, lego/lego_mlir.py:105-107)."""
+    mod = dsl_transpose.row_sums(128, 48)
+    text = mod.source
+    assert "float carry" in text and "= 0.0;" in text
+    body = text[text.index("for (unsigned"):]
+    assert body.index("const float next") < body.index("carry", body.index("const float next") + 20)
+    assert "+= 1" in body and "< 48" in body
+    # two carried values swap through temporaries, not through each other
+    from lego_amd.lego_hip import HipTensor, printer
+    from lego_amd.lego import OrderBy, Row
+
+    @printer.generate_hip(name="swap")
+    def module():
+        T = HipTensor(OrderBy(Row(64)).TileBy([64]), "f32")
+
+        @printer.generate_gpu_kernel([T], [T], (1, 1, 1), (64, 1, 1))
+        def kernel(_):
+            tX = printer.get_thread_linear_index()
+
+            @printer.generate_loop(OrderBy(Row(3)).TileBy([3]), iter_args=[1.0, 2.0])
+            def swap(pargs, _, carried):
+                return carried[1], carried[0]
+            a, b = swap()
+            T[tX] = a - b
+    lines = [ln.strip() for ln in module.source.splitlines()]
+    first = next(i for i, ln in enumerate(lines) if ln.startswith("const float next"))
+    assert lines[first + 1].startswith("const float next") and lines[first + 2].startswith("carry")
+    with pytest.raises(ValueError):
+        @printer.generate_hip(name="bad")
+        def bad():
+            T = HipTensor(OrderBy(Row(64)).TileBy([64]), "f32")
+
+            @printer.generate_gpu_kernel([T], [T], (1, 1, 1), (64, 1, 1))
+            def kernel(_):
+                @printer.generate_loop(OrderBy(Row(3)).TileBy([3]), iter_args=[1.0, 2.0])
+                def loop(pargs, _, carried):
+                    return carried[0]
+                loop()

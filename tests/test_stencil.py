@@ -145,6 +145,42 @@ def test_gpu_laplacian_matches_oracle(n, radius, bricks):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("kind,radius", [("f3d", 1), ("f3d", 3), ("laplacian", 1), ("laplacian", 3)])
+def test_gpu_stencils_full_size_match_oracle_on_slabs(kind, radius):
+    """The reference's size, 384^3, both storage orders, against the float64 oracle on three slabs of 16
+    planes (the first, one across the middle of the brick grid, the last): the oracle of a slab widened
+    by the radius equals the oracle of the cube on the slab's own planes."""
+    from lego_amd import ops
+    print(f"{kind} 384^3 radius {radius} against the oracle on slabs", flush=True)
+    n = 384
+    x = torch.rand(n, n, n, generator=torch.Generator().manual_seed(51 + radius)) * 2 - 1
+    if kind == "f3d":
+        c = torch.from_numpy(_coefficients(radius))
+        call, oracle, tol = ops.stencil_f3d, ok.stencil_f3d, 2e-5 * (2 * radius + 1) ** 3
+    else:
+        c = torch.tensor([-6.0, 1.0, 0.5, 0.25])[:radius + 1].contiguous()
+        call, oracle, tol = ops.stencil_laplacian, ok.stencil_laplacian, 1e-5
+    order = ok.bricks_order(n)
+    rowmajor = call(x.cuda(), c.cuda(), radius, False).cpu()
+    bricks = _from_bricks(call(_to_bricks(x, order).cuda(), c.cuda(), radius, True).cpu(), order)
+    assert torch.equal(rowmajor, bricks)
+    for lo, hi in ((0, 16), (184, 200), (n - 16, n)):
+        a, b = max(0, lo - radius), min(n, hi + radius)
+        want = torch.from_numpy(oracle(x[a:b].numpy(), c.numpy(), radius)).float()
+        # planes of the slab that are boundary planes of the widened slab but not of the cube are not the cube's
+        keep = slice(lo - a, hi - a)
+        got = rowmajor[lo:hi]
+        ref = want[keep]
+        if lo == 0:
+            assert got[:radius].abs().max().item() == 0          # the cube's own boundary planes are not written
+            got, ref = got[radius:], ref[radius:]
+        if hi == n:
+            assert got[-radius:].abs().max().item() == 0
+            got, ref = got[:-radius], ref[:-radius]
+        assert (got - ref).abs().max().item() <= tol, (lo, hi)
+
+
+@pytest.mark.gpu
 def test_gpu_stencils_full_size_agree_between_layouts():
     """The reference's size, 384^3: both storage orders give the same field, bit for bit (the
     arithmetic of a point does not depend on where its neighbours are stored)."""
