@@ -58,6 +58,9 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--sustain", type=float, default=0.0, metavar="SECONDS",
+                    help="after timing the 8192^3 GEMM, keep launching it back to back for this long (for sampling "
+                         "socket power and clocks with amd-smi from another process) and report the sustained rate")
     ap.add_argument("--only", default="", help="comma list of configs to time (c1,c2,c3,c4,c5,extra,apps); "
                     "c2 is always timed; 'extra' adds LayerNorm backward and the other GEMM layouts and element "
                     "types, 'apps' the stencil, Needleman-Wunsch and LUD programs")
@@ -286,6 +289,15 @@ def main():
                                            vendor_library_tflops_b_moved_128_bytes=fl4 / lib_ms_s / 1e9,
                                            note="vendor_library = torch.matmul (hipBLASLt) on the same buffers")
         del b4s, b4s_buf
+        if ns.sustain > 0:
+            for name, fn in (("sustained", gm), ("vendor_library_sustained", lambda: torch.matmul(a4, b4, out=c4))):
+                per = []
+                t_end = time.perf_counter() + ns.sustain
+                while time.perf_counter() < t_end:
+                    per.append(timed(fn, steps=100, warmup=1))
+                kernels["c4_gemm_f16_8192"][name + "_tflops"] = fl4 / (sum(per) / len(per)) / 1e9
+                kernels["c4_gemm_f16_8192"][name + "_seconds"] = ns.sustain
+                time.sleep(1.0)      # an idle second between the two, visible in the power samples
         if not ns.skip_cpu:
             from oracle import kernels as ok4
             a4c, b4c = a4[:1024].cpu(), b4.cpu()
