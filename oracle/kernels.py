@@ -157,3 +157,15 @@ def stencil_laplacian(x, c, radius):
                             + x[i, j, sh(k, a)] + x[i, j, sh(k, -a)])
     out[core] = acc
     return out
+
+
+def lud(a):
+    """LU decomposition without pivoting (Doolittle, unit lower triangle), what Rodinia's
+    ``lud_base`` computes (the reference's CPU check, benchmarks/cuda/lud/lud.cu with common.c), in
+    float64: returns one matrix with L below the diagonal and U on and above it."""
+    m = np.array(a, dtype=np.float64)
+    n = m.shape[0]
+    for k in range(n - 1):
+        m[k + 1:, k] /= m[k, k]
+        m[k + 1:, k + 1:] -= np.outer(m[k + 1:, k], m[k, k + 1:])
+    return m
