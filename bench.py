@@ -58,6 +58,9 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
+                    help="untimed device time of back-to-back launches before every timed region (0 for counter runs, "
+                         "whose values do not depend on the clocks)")
     ap.add_argument("--sustain", type=float, default=0.0, metavar="SECONDS",
                     help="after timing the 8192^3 GEMM, keep launching it back to back for this long (for sampling "
                          "socket power and clocks with amd-smi from another process) and report the sustained rate")
@@ -97,7 +100,7 @@ def main():
         stop.record()
         torch.cuda.synchronize()
         per_call = start.elapsed_time(stop) / max(1, warmup)
-        for _ in range(min(5000, int(SETTLE_MS / max(per_call, 1e-3)) + 1)):
+        for _ in range(min(5000, int(ns.settle_ms / max(per_call, 1e-3)) + 1) if ns.settle_ms > 0 else 0):
             fn()
         start.record()
         for _ in range(steps):

@@ -41,8 +41,10 @@ def test_benchmark_reads_the_committed_traffic_summary():
     row = next(line for line in text.splitlines() if line.startswith(bench.HEADLINE_KERNEL + " "))
     fetch_kib, write_kib, scaled, algorithmic = [int(t) for t in row.split(")", 1)[1].split()[:4]]
     assert got == scaled
-    # the scaled figure is what the counters say: FETCH_SIZE counts half of every 128-byte request at
-    # this access width (the copy calibration in the same file reads 262150 KiB for 512 MiB: factor
-    # 2 * 262144 / 262150), WRITE_SIZE all of it
-    assert abs(scaled - (2.0 * 262144 / 262150 * fetch_kib + write_kib) * 1024) <= 4096
+    # the scaled figure is what the counters say, each scaled by what the same counter reads for the plain
+    # 512 MiB copy in the same file (FETCH_SIZE counts half of every 128-byte request at this access width)
+    import re
+    cal_fetch, cal_write = (int(v) for v in re.search(r"reads FETCH_SIZE=(\d+) KiB and writes WRITE_SIZE=(\d+) KiB", text).groups())
+    known = 512 * 1024
+    assert abs(scaled - (known / cal_fetch * fetch_kib + known / cal_write * write_kib) * 1024) <= 4096
     assert algorithmic == 2 * 16384 * 16384 * 2
