@@ -21,6 +21,7 @@ from ..lego import BitXor, Col, GenP, OrderBy, Row
 from .common import BANNER, Emitted, code, idx, size, template, tidy
 
 XCDS = 8
+CUS = 256      # MI355X: 8 XCDs of 32 CUs
 MAX_GROUPS = 64
 
 
@@ -289,10 +290,23 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
         c_out_row=code(c_out[0]), c_out_pair=code(c_out[1]),
         c_stage_load=code(tidy(4 * Cs_L[cr, 2 * cp], rng) - 4 * (cr % 2)),
         c_goff=code(tidy(C_L[pid_m, pid_n, wm * WM + cr, wn * WN + 8 * cp], rng)),
-        xcd_pid=code(tidy(xcd_remap(per_xcd, wg), {wg: (0, per_xcd * XCDS)})),
+        xcd_pid=code(tidy(xcd_remap(per_xcd, wg), {wg: (0, per_xcd * XCDS)})), CUS=CUS,
         pid_m=code(pm_e), pid_n=code(pn_e),
     )
     return params
+
+
+def class_order(p, count, first_wg, cus=CUS, xcds=XCDS):
+    """Place, among ``count`` tiles of equal depth, of the workgroup that is number ``p`` of those working on
+    them (``first_wg``: the id of number 0), with integers, as the grouped kernels compute it: rounds of
+    ``cus`` workgroups in order, and within a round ``xcd_remap`` over the round's length when ids and XCDs
+    line up (``first_wg`` and the length multiples of ``xcds``)."""
+    wg = p % cus
+    round0 = p - wg
+    length = cus if round0 + cus <= count else count - round0
+    if first_wg % xcds or length % xcds:
+        return p
+    return round0 + int(xcd_remap(length // xcds, wg))
 
 
 def split_order(split, wg):
@@ -320,7 +334,7 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
         split, swg, ti, hf = size("split"), idx("swg"), idx("pid_m"), idx("half")
         tile_e, half_e = (tidy(e, {swg: (0, 2 * split)}) for e in split_order(split, swg))
         params.update(half_ns=hns, HBM=bm // 2,
-                      split_layout="OrderBy(Row(split, 2)).TileBy([split, 2]).inv(wg - whole)",
+                      split_layout="OrderBy(Row(split, 2)).TileBy([split, 2]).inv(s)",
                       split_tile=code(tile_e), split_half=code(half_e),
                       # rows of halves in place of rows of tiles: one more level under the tile row
                       half_pid_m=code(tidy(OrderBy(Row(size("num_pid_m"), 2)).TileBy([size("num_pid_m"), 2])[ti, hf],

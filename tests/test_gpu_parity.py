@@ -691,6 +691,25 @@ def test_grouped_gemm_split_matches_whole_tiles_bit_for_bit(ops):
             assert torch.equal(c, w)
 
 
+@pytest.mark.parametrize("split", [0, 40, 300])
+def test_grouped_gemm_launch_order_over_depth_classes(ops, split):
+    """Workgroup ids are dealt to tiles per class of equal depth, in rounds of 256 with a contiguous run per
+    XCD: a class that starts at a flat index that is not a multiple of 8 (3 tiles come before it), one of
+    289 + 20 tiles (a whole round, then a remainder of 53 that is not a multiple of 8), one of 72 + 24 (a
+    remainder that is), and the same with the last tiles as halves, so that the whole tiles of a class stop
+    and its halves start in the middle of it.  Every tile must be computed exactly once: against the oracle."""
+    print(f"grouped gemm launch order over depth classes, split {split}", flush=True)
+    g = _gen(61)
+    shapes = [(768, 256, 192), (4352, 4352, 128), (1024, 1280, 128), (2048, 2304, 64), (1536, 1024, 64)]
+    A = [(torch.randn(m, k, generator=g) / math.sqrt(k)).half() for m, n, k in shapes]
+    B = [(torch.randn(k, n, generator=g) / math.sqrt(k)).half() for m, n, k in shapes]
+    want = ok.grouped_gemm(A, B)
+    got = _grouped_call("lego_hip_grouped_gemm_f16_split", [a.cuda() for a in A], [b.cuda() for b in B], split)
+    for c, w in zip(got, want):
+        assert _rel_err(c.cpu(), w) <= 1e-2
+        assert (c.cpu().float() - w.float()).abs().max().item() <= 1e-2
+
+
 def test_gemm_headline_shape_8192_cubed(ops):
     """Config 4 at full size: 1024 tiles, 128 k-steps each, operands 128 MiB apart as two consecutive
     allocations are.  Two 256-row panels (the first tile row and one in the middle of the launch order's

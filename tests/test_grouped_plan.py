@@ -37,12 +37,26 @@ def _coverage(sizes, split):
     total = int(ends[-1])
     whole = total - split
     seen = [np.zeros((2 * tm, tn), dtype=int) for tm, tn in tiles]
+    depth = [sizes[g][2] for g in order]
+
+    def depth_class(tile):
+        """Flat tile range of the problems whose depth is that of the problem holding `tile`."""
+        s = int(np.searchsorted(ends, tile, side="right"))
+        first = min(q for q in range(len(order)) if depth[q] == depth[s])
+        last = max(q for q in range(len(order)) if depth[q] == depth[s])
+        return (int(ends[first - 1]) if first else 0), int(ends[last])
+
     for wg in range(total + split):
         if wg < whole:
-            tile, half = wg, None
+            cb, ce = depth_class(wg)
+            tile, half = cb + gemm.class_order(wg - cb, min(ce, whole) - cb, cb), None
         else:
-            t, half = gemm.split_order(split, wg - whole)               # Row(split, 2).inv(wg - whole)
-            tile = whole + int(t)
+            cb, ce = depth_class(whole + (wg - whole) // 2)
+            first_tile = max(cb, whole)
+            first_wg = whole + 2 * (first_tile - whole)
+            swg = gemm.class_order(wg - first_wg, 2 * (ce - first_tile), first_wg)
+            t, half = gemm.split_order(ce - first_tile, swg)            # Row(tiles, 2).inv(swg)
+            tile = first_tile + int(t)
         s = int(np.searchsorted(ends, tile, side="right"))
         pid = tile - (int(ends[s - 1]) if s else 0)
         npm, npn = tiles[s]
@@ -57,7 +71,9 @@ def _coverage(sizes, split):
 
 
 @pytest.mark.parametrize("sizes", [C5, [(256, 256, 64)], [(1000, 776, 192), (520, 264, 128), (136, 512, 64)],
-                                   [(2048, 2048, 512)] * 5, [(4096, 4096, 4096), (512, 512, 64)]])
+                                   [(2048, 2048, 512)] * 5, [(4096, 4096, 4096), (512, 512, 64)],
+                                   [(768, 256, 192), (4352, 4352, 128), (1024, 1280, 128), (2048, 2304, 64),
+                                    (1536, 1024, 64)]])
 def test_every_block_of_c_is_computed_once(sizes):
     kind, total, split = _plan(sizes)
     assert total == sum(-(-m // 256) * -(-n // 256) for m, n, _ in sizes)
