@@ -124,9 +124,9 @@ def test_fragments_receive_the_right_elements(dtype, bk, tile, variant):
 @pytest.mark.parametrize("tile", [256, 128])
 @pytest.mark.parametrize("variant", ["nn", "nt", "tn", "tt"])
 def test_ragged_edges_skip_exactly_what_lies_outside(variant, tile):
-    """The EDGE instantiation guards every memory->LDS chunk with ``edge0 + X*step < rem``.  For a
-    tile with ``rem`` valid rows (columns), replay the guards: every chunk that passes must lie
-    inside the operand, and every chunk with data of a valid row (column) must pass."""
+    """The EDGE instantiation runs memory->LDS instruction ``x`` under the mask of the lanes with
+    ``edge0 + x*step < rem``.  For a tile with ``rem`` valid rows (columns), replay the masks: every chunk that
+    passes must lie inside the operand, and every chunk with data of a valid row (column) must pass."""
     ta, tb = variant[0] == "t", variant[1] == "t"
     bk = 64
     unit, _ = gemm.emit(bm=tile, bn=tile, bk=bk, trans_a=ta, trans_b=tb, with_grouped=False)
@@ -137,7 +137,7 @@ def test_ragged_edges_skip_exactly_what_lies_outside(variant, tile):
         step = _grab(text, r"%s_src_step = \d \* \((.*?)\)[,;]" % role)
         edge0 = _grab(text, r"const unsigned a_edge0 = (.*), b_edge0 = .*;") if role == "a" else \
             _grab(text, r"const unsigned a_edge0 = .*, b_edge0 = (.*);")
-        estep = int(_grab(text, r"%s_edge0 \+ \(.*?\) \* \((\d+)\) < %s_rem" % (role, "m" if role == "a" else "n")))
+        estep = int(_grab(text, r"%s_edge0 \+ x \* \((\d+)\) < %s_rem" % (role, "m" if role == "a" else "n")))
         for rem in (r for r in (8, 40, 120, 128, 200, 248) if r <= tile):
             rows_total = rem                     # the operand ends where the tile's valid part ends
             sizes = dict(M=rows_total, N=rows_total, K=K)
@@ -164,8 +164,9 @@ def test_ragged_edges_skip_exactly_what_lies_outside(variant, tile):
 @pytest.mark.parametrize("dtype,bk", [("f16", 64), ("e5m2", 128)])
 @pytest.mark.parametrize("variant", ["nn", "tt"])
 def test_last_k_tile_zeroes_exactly_what_lies_past_k(dtype, bk, variant):
-    """The EDGE instantiation guards every slot of the last k-tile with ``k0 + X*step >= klim``: such a slot
-    is written as zeros, the others are fetched.  For every ``klim`` in whole chunks, replay the guards
+    """In the last k-tile of a ragged K the EDGE instantiation keeps a lane in instruction ``x``'s mask while
+    ``k0 + x*step < klim``: the slots of the other lanes are written as zeros, once, instead of being fetched.
+    For every ``klim`` in whole chunks, replay the guards
     over all slots: a slot is zeroed exactly when the chunk that the layout puts there starts at or past
     ``klim`` (chunks never straddle it), so the tile ends up holding the operand's k-values below
     ``klim`` and zeros above."""
@@ -181,7 +182,7 @@ def test_last_k_tile_zeroes_exactly_what_lies_past_k(dtype, bk, variant):
     for role, rows_total, kmajor, k0_text in (("a", 512, not ta, k0s[0]), ("b", 512, tb, k0s[1])):
         src0 = _grab(text, r"const unsigned %s_src0 = \d \* \((.*)\);" % role)
         step = _grab(text, r"%s_src_step = \d \* \((.*?)\)[,;]" % role)
-        kstep = int(_grab(text, r"%s_k0 \+ \(.*?\) \* \((\d+)\) >= klim_nx" % role))
+        kstep = int(_grab(text, r"%s_k0 \+ x \* \((\d+)\) < klim_nx" % role))
         iters = tile * bk // epc // 256
         for klim in range(epc, bk + 1, epc):
             zeroed, fetched = set(), set()
