@@ -25,7 +25,7 @@ OBJ_DIR = LIB_DIR / "obj"
 
 # the tilings the library is built with
 # Per element type, in order of preference: the fastest tiling for shapes that its windows
-# divide, a wide macro tile in skewed ("diag") order, a 64x64 one for shapes the wide tile
+# divide (then the same in smaller windows), a wide macro tile in skewed ("diag") order, a 64x64 one for shapes the wide tile
 # does not divide, and the wide tile with edge tests for shapes in whole 16-byte vectors.
 TRANSPOSE = {
     "f32": [dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 64, 8), max_bytes=256 << 20),
@@ -34,6 +34,8 @@ TRANSPOSE = {
             dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag"),
             dict(dtype="f32", tile=(32, 32), group=(2, 4), order="diag", edge=True)],
     "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 128, 8)),
+            dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 64, 8)),
+            dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 32, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag"),
             dict(dtype="f16", tile=(64, 64), group=(1, 1), order="diag"),
             dict(dtype="f16", tile=(64, 64), group=(2, 2), order="diag", edge=True)],
@@ -45,6 +47,8 @@ ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f16", True, 8
            ("f16", True, 16), ("f32", True, 16), ("f16", False, 16), ("f32", False, 16),
            ("bf16", True, 1), ("bf16", True, 4), ("bf16", True, 16), ("bf16", False, 1), ("bf16", False, 4),
            ("bf16", False, 16)]
+# (element type, lanes per row): teams of a part of a wave for rows of at most that many 16-byte vectors
+ROWWISE_SHORT = [(d, lanes) for d in ("f16", "bf16", "f32") for lanes in (16, 32)]
 # LayerNorm launches of many rows: this many workgroups that stage gamma and beta in LDS and walk the rows
 ROWWISE_STREAM_WGS = {("f16", True, 8): 512}
 ROWWISE_DEFAULT_WAVES = 4
@@ -75,6 +79,7 @@ def collect():
             tmeta.setdefault(dtype, []).append(meta)
     units.append(transpose.emit_any())
     units += [rowwise.emit(w, dtype, vec, stream_wgs=ROWWISE_STREAM_WGS.get((dtype, vec, w), 0)) for dtype, vec, w in ROWWISE]
+    units += [rowwise.emit(1, dtype, True, team_lanes=lanes) for dtype, lanes in ROWWISE_SHORT]
     units.append(rowwise.emit_long())
     for dtype in GEMM_DTYPES:
         for ta in (False, True):
@@ -120,6 +125,10 @@ def collect():
         tag = dtype if vec else dtype + "s"
         h += [f"hipError_t lego_softmax_{tag}_w{w}_launch(const void*, void*, int, int, hipStream_t);",
               f"hipError_t lego_layernorm_fwd_{tag}_w{w}_launch(const void*, void*, const void*, const void*, "
+              "float*, float*, int, int, float, hipStream_t);"]
+    for dtype, lanes in ROWWISE_SHORT:
+        h += [f"hipError_t lego_softmax_{dtype}_l{lanes}_launch(const void*, void*, int, int, hipStream_t);",
+              f"hipError_t lego_layernorm_fwd_{dtype}_l{lanes}_launch(const void*, void*, const void*, const void*, "
               "float*, float*, int, int, float, hipStream_t);"]
     h += [f"hipError_t lego_softmax_long_{d}_launch(const void*, void*, int, int, hipStream_t);" for d in rowwise.ELEMENTS]
     h += [

@@ -95,7 +95,9 @@ int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per
   if (!usable(x) || !usable(y)) return kInvalid;
   if (M <= 0 || N <= 0 || N % 8 || N > LEGO_ROWWISE_MAX_N) return kInvalid;
   switch (waves_per_row) {
-    case 1: return ok_or(lego_softmax_f16_w1_launch(x, y, M, N, as_stream(stream)));
+    case 1:   // rows of at most 16 or 32 vectors: several rows per wave
+      return ok_or((N <= 128 ? lego_softmax_f16_l16_launch : N <= 256 ? lego_softmax_f16_l32_launch : lego_softmax_f16_w1_launch)(
+          x, y, M, N, as_stream(stream)));
     case 2: return ok_or(lego_softmax_f16_w2_launch(x, y, M, N, as_stream(stream)));
     case 4: return ok_or(lego_softmax_f16_w4_launch(x, y, M, N, as_stream(stream)));
     case 8: return ok_or(lego_softmax_f16_w8_launch(x, y, M, N, as_stream(stream)));
@@ -124,7 +126,9 @@ int lego_hip_softmax_f32(const void* x, void* y, int M, int N, void* stream)
   if (N % 4)   // ragged rows
     return ok_or((long_row ? lego_softmax_f32s_w16_launch : N <= 1024 ? lego_softmax_f32s_w1_launch
                                                                       : lego_softmax_f32s_w4_launch)(x, y, M, N, as_stream(stream)));
-  if (N <= 1024) return ok_or(lego_softmax_f32_w1_launch(x, y, M, N, as_stream(stream)));
+  if (N <= 1024)   // rows of at most 16 or 32 vectors: several rows per wave
+    return ok_or((N <= 64 ? lego_softmax_f32_l16_launch : N <= 128 ? lego_softmax_f32_l32_launch : lego_softmax_f32_w1_launch)(
+        x, y, M, N, as_stream(stream)));
   return ok_or((long_row ? lego_softmax_f32_w16_launch : lego_softmax_f32_w4_launch)(x, y, M, N, as_stream(stream)));
 }
 
@@ -135,7 +139,10 @@ int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const 
   if (!usable(x) || !usable(y) || !usable(w) || !usable(b) || mean == nullptr || rstd == nullptr) return kInvalid;
   if (M <= 0 || N <= 0 || N % 8 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
   switch (waves_per_row) {
-    case 1: return ok_or(lego_layernorm_fwd_f16_w1_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+    case 1:   // rows of at most 16 or 32 vectors: several rows per wave
+      return ok_or((N <= 128 ? lego_layernorm_fwd_f16_l16_launch : N <= 256 ? lego_layernorm_fwd_f16_l32_launch
+                                                                         : lego_layernorm_fwd_f16_w1_launch)(
+          x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
     case 2: return ok_or(lego_layernorm_fwd_f16_w2_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
     case 4: return ok_or(lego_layernorm_fwd_f16_w4_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
     case 8: return ok_or(lego_layernorm_fwd_f16_w8_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
@@ -167,7 +174,10 @@ int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void
     return ok_or((long_row ? lego_layernorm_fwd_f32s_w16_launch : N <= 1024 ? lego_layernorm_fwd_f32s_w1_launch
                                                                             : lego_layernorm_fwd_f32s_w4_launch)(
         x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
-  if (N <= 1024) return ok_or(lego_layernorm_fwd_f32_w1_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+  if (N <= 1024)
+    return ok_or((N <= 64 ? lego_layernorm_fwd_f32_l16_launch : N <= 128 ? lego_layernorm_fwd_f32_l32_launch
+                                                                      : lego_layernorm_fwd_f32_w1_launch)(
+        x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
   return ok_or((long_row ? lego_layernorm_fwd_f32_w16_launch : lego_layernorm_fwd_f32_w4_launch)(
       x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
 }
@@ -180,6 +190,7 @@ int lego_hip_softmax_bf16(const void* x, void* y, int M, int N, void* stream)
   if (N % 8)   // ragged rows
     return ok_or((wpr == 16 ? lego_softmax_bf16s_w16_launch : wpr == 1 ? lego_softmax_bf16s_w1_launch
                                                                        : lego_softmax_bf16s_w4_launch)(x, y, M, N, as_stream(stream)));
+  if (N <= 256) return ok_or((N <= 128 ? lego_softmax_bf16_l16_launch : lego_softmax_bf16_l32_launch)(x, y, M, N, as_stream(stream)));
   return ok_or((wpr == 16 ? lego_softmax_bf16_w16_launch : wpr == 1 ? lego_softmax_bf16_w1_launch
                                                                     : lego_softmax_bf16_w4_launch)(x, y, M, N, as_stream(stream)));
 }
@@ -193,6 +204,9 @@ int lego_hip_layernorm_fwd_bf16(const void* x, void* y, const void* w, const voi
   if (N % 8)   // ragged rows
     return ok_or((wpr == 16 ? lego_layernorm_fwd_bf16s_w16_launch : wpr == 1 ? lego_layernorm_fwd_bf16s_w1_launch
                                                                              : lego_layernorm_fwd_bf16s_w4_launch)(
+        x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+  if (N <= 256)
+    return ok_or((N <= 128 ? lego_layernorm_fwd_bf16_l16_launch : lego_layernorm_fwd_bf16_l32_launch)(
         x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
   return ok_or((wpr == 16 ? lego_layernorm_fwd_bf16_w16_launch : wpr == 1 ? lego_layernorm_fwd_bf16_w1_launch
                                                                           : lego_layernorm_fwd_bf16_w4_launch)(

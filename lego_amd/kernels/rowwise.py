@@ -27,16 +27,22 @@ LONG_ROW_WAVES = 16
 VPTS = (1, 2, 4, 8, 16, 32, 64)
 
 
-def emit(waves_per_row=1, dtype="f16", vectorised=True, seq_max_wpr=4, prefetch_max_wpr=4, stream_wgs=0):
+def emit(waves_per_row=1, dtype="f16", vectorised=True, seq_max_wpr=4, prefetch_max_wpr=4, stream_wgs=0, team_lanes=None):
     """One translation unit: every register footprint ``V`` of one (waves per row, element type,
     access width) combination.  ``vectorised=False`` emits the kernels that take rows of any length
     and alignment (the reference's own softmax test is 1823 x 781): the elements before a row's
-    first 16-byte boundary and after its last whole vector go one per lane, the rest as vectors."""
+    first 16-byte boundary and after its last whole vector go one per lane, the rest as vectors.
+    ``team_lanes`` (16 or 32) makes teams of a part of a wave for rows of at most ``team_lanes`` vectors:
+    a row of 128 halves in a wave of its own would leave 48 of 64 lanes without a vector."""
     WPR = waves_per_row
     elt, esize = ELEMENTS[dtype]
     EPV = 16 // esize
     tag = dtype if vectorised else dtype + "s"
     TEAM = 64 * WPR
+    wtag = f"w{WPR}"
+    if team_lanes:
+        assert WPR == 1 and vectorised and team_lanes in (16, 32)
+        TEAM, wtag = team_lanes, f"l{team_lanes}"
     threads = max(THREADS, TEAM)
     RPW = threads // TEAM                       # rows per workgroup
     # register footprints: a lane keeps V*EPV fp32 values, at most 128; the sixteen-wave team only
@@ -62,8 +68,8 @@ def emit(waves_per_row=1, dtype="f16", vectorised=True, seq_max_wpr=4, prefetch_
     stream_row = tidy(OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])[step, wg], {step: (0, STEPS), wg: (0, G)})
 
     params = dict(
-        banner=BANNER, WPR=WPR, TEAM=TEAM, RPW=RPW, THREADS=threads,
-        VPTS=[vp for vp in VPTS if vp * EPV <= 128 and lo < vp * TEAM * EPV <= hi],
+        banner=BANNER, WPR=WPR, TEAM=TEAM, RPW=RPW, THREADS=threads, WTAG=wtag, SHUFFLE=min(TEAM, 64),
+        VPTS=[1] if team_lanes else [vp for vp in VPTS if vp * EPV <= 128 and lo < vp * TEAM * EPV <= hi],
         dtype=dtype, elt=elt, EPV=EPV, ESIZE=esize, RAGGED=not vectorised, tag=tag,
         SEQ_MAX_WPR=seq_max_wpr, PREFETCH_MAX_WPR=prefetch_max_wpr,
         STREAM=vectorised and RPW == 1 and WPR < LONG_ROW_WAVES and stream_wgs > 0, STREAM_WGS=stream_wgs,
@@ -76,8 +82,8 @@ def emit(waves_per_row=1, dtype="f16", vectorised=True, seq_max_wpr=4, prefetch_
         vec=code(vec_e), vec_off=code(vec_off), stat_off=code(stat),
     )
     text = template("rowwise.hip.j2").render(**params)
-    return Emitted(f"rowwise_{tag}_w{WPR}.hip", text,
-                   [f"lego_softmax_{tag}_w{WPR}_launch", f"lego_layernorm_fwd_{tag}_w{WPR}_launch"])
+    return Emitted(f"rowwise_{tag}_{wtag}.hip", text,
+                   [f"lego_softmax_{tag}_{wtag}_launch", f"lego_layernorm_fwd_{tag}_{wtag}_launch"])
 
 
 def emit_long():

@@ -29,6 +29,8 @@ def _gen(seed):
     (torch.float16, 64, 256), (torch.float16, 320, 768),
     (torch.float32, 2048, 1024), (torch.float32, 4096, 3072),    # windowed cache-resident fp32 tiling
     (torch.float16, 8192, 2048),                    # one window of the windowed tile order
+    (torch.float16, 4096, 6144), (torch.float16, 12288, 2048),    # windows of 64 x 8 macro tiles: one, and three by one
+    (torch.float16, 2048, 4096), (torch.float16, 6144, 2048),     # windows of 32 x 8: one by two, three by one
 ])
 def test_transpose_matches_oracle(ops, dtype, rows, cols):
     print(f"transpose {dtype} {rows}x{cols}", flush=True)
@@ -357,6 +359,31 @@ def test_layernorm_backward_fp32(ops, M, N):
     assert (xd.grad.cpu().double() - xc.grad).abs().max().item() <= 2e-5
     assert (wd.grad.cpu().double() - wc.grad).abs().max().item() <= 2e-5 * max(1.0, wc.grad.abs().max().item())
     assert (bd.grad.cpu().double() - bc.grad).abs().max().item() <= 2e-5 * max(1.0, bc.grad.abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M,N", [(1, 8), (37, 24), (300, 64), (77, 120), (1000, 128), (41, 136), (513, 248), (260, 256)])
+def test_short_rows_share_a_wave(ops, dtype, M, N):
+    """Rows of at most 16 or 32 vectors are dealt 4 or 2 to a wave (teams of 16 or 32 lanes, 16 or 8 rows per
+    workgroup, LayerNorm two rows per team): row counts that leave teams and workgroups partly empty, row
+    lengths at, between and just past the team sizes of both element widths."""
+    print(f"short rows {dtype} {M}x{N}", flush=True)
+    g = _gen(71)
+    x = (2.0 * torch.randn(M, N, generator=g)).to(dtype)
+    w = (1 + 0.1 * torch.randn(N, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(N, generator=g)).to(dtype)
+    got = ops.softmax(x.cuda()).cpu()
+    tol = {torch.float16: TOL, torch.bfloat16: 2.0 ** -9 + 1e-6, torch.float32: 1e-6}[dtype]
+    assert (got.float() - ok.softmax(x).float()).abs().max().item() <= tol
+    assert (got.float().sum(-1) - 1).abs().max().item() <= {torch.float32: 1e-5}.get(dtype, 2e-2)
+    y, mean, rstd = ops.layer_norm_fwd(x.cuda(), w.cuda(), b.cuda(), 1e-5)
+    _, want_mean, want_rstd = ok.layernorm_fwd(x, w, b, 1e-5)
+    assert (mean.cpu() - want_mean).abs().max().item() <= 1e-5
+    assert ((rstd.cpu() - want_rstd).abs() <= 1e-4 * want_rstd.abs()).all()
+    if dtype == torch.float32:
+        assert (y.cpu() - ok.layernorm_fwd_unrounded(x, w, b)).abs().max().item() <= 2e-5
+    else:
+        _assert_layernorm_forward(y, x, w, b)
 
 
 @pytest.mark.parametrize("M,N", [(5, 8), (9, 781), (33, 2048), (64, 8192), (3, 8191), (4, 20000), (2, 32768), (2, 50257)])
