@@ -122,6 +122,19 @@ int lego_hip_gemm_bf16_ex(const void* a, const void* b, void* c, int M, int N, i
  * `accumulator.to(tl.float16)` into a float16 tensor whatever its operands' type, matmul_sympy.py:136, 203). */
 int lego_hip_gemm_bf16_f16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                               int activation, void* stream);
+/* The same products (element: 0 = fp16, 1 = bfloat16, 4 = bfloat16 operands with fp16 result) with room for partial
+ * sums.  A product of few tiles -- a skinny operand (16 x 8192 x 8192), a long K (256 x 256 x 65536) -- leaves most
+ * CUs idle with one workgroup per tile and cannot pull its operands through the chip; with a workspace the k-tiles
+ * of every tile are dealt to several workgroups, which leave fp32 sums there, and a second kernel adds them in a
+ * fixed order (deterministic), applies the activation and stores C.  lego_hip_gemm_workspace_bytes gives the size
+ * the call uses for a shape (0: it gains nothing from parts).  The workspace is scratch: 16-byte aligned device
+ * memory, contents undefined on entry and exit, not to be shared by calls that may overlap.  With a null or short
+ * workspace, or a shape outside the tiled kernels, the call is lego_hip_gemm_*_ex.  No counterpart in the
+ * reference, whose matmul has one program per tile (matmul_sympy.py:57-65). */
+int lego_hip_gemm_workspace_bytes(int M, int N, int K, unsigned long long* bytes);
+int lego_hip_gemm_ex_ws(int element, const void* a, const void* b, void* c, int M, int N, int K, int trans_a,
+                        int trans_b, int activation, void* workspace, unsigned long long workspace_bytes,
+                        void* stream);
 /* 8-bit floating-point operands, fp32 accumulation, fp16 result: the reference's fp8 path casts
  * both operands to float8_e5m2 and stores fp16 (matmul_sympy.py:346-364, 203).  format 0 = OCP
  * e4m3 (torch.float8_e4m3fn), 1 = OCP e5m2 (torch.float8_e5m2); a and b hold one byte per

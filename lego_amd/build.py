@@ -95,7 +95,7 @@ def collect():
                 if dtype in GEMM_SMALL_DTYPES:
                     gs, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK[dtype], bm=GEMM_SMALL_TILE, bn=GEMM_SMALL_TILE),
                                       trans_a=ta, trans_b=tb, dtype=dtype,
-                                      with_grouped=dtype == "f16" and not (ta or tb))
+                                      with_grouped=dtype == "f16" and not (ta or tb), with_splitk=True)
                     units.append(gs)
     units.append(gemm.emit_any())
     lb, mlb = layernorm_bwd.emit()
@@ -155,6 +155,8 @@ def collect():
     h += [f"hipError_t lego_gemm_{d}_{v}{t}_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);"
           for d in GEMM_DTYPES for v in ("nn", "nt", "tn", "tt")
           for t in ("", f"_t{GEMM_SMALL_TILE}x{GEMM_SMALL_TILE}") if not t or d in GEMM_SMALL_DTYPES]
+    h += [f"hipError_t lego_gemm_{d}_{v}_t{GEMM_SMALL_TILE}x{GEMM_SMALL_TILE}_splitk_launch(const void*, const void*, void*, int, int, int, int, "
+          "int, float*, hipStream_t);" for d in GEMM_SMALL_DTYPES for v in ("nn", "nt", "tn", "tt")]
     h += [
           "hipError_t lego_grouped_gemm_f16_launch(const void* const*, const void* const*, void* const*, "
           "const int*, int, hipStream_t);",

@@ -327,6 +327,19 @@ int gemm_ex(const GemmKernels& k, int element, const void* a, const void* b, voi
   return ok_or(by_layout[(trans_a ? 2 : 0) + (trans_b ? 1 : 0)](a, b, c, M, N, K, activation, as_stream(stream)));
 }
 
+// Parts along K for a product of few tiles (1: one workgroup per tile does it all): enough parts for two
+// workgroups of 128 x 128 tiles per CU, at least four k-tiles each.
+int splitk_parts(int M, int N, int K, int bk)
+{
+  const long tiles = static_cast<long>((M + 127) / 128) * ((N + 127) / 128), depth = (K + bk - 1) / bk;
+  if (tiles > 128 || depth < 8) return 1;
+  long parts = (512 + tiles - 1) / tiles;
+  if (parts > depth / 4) parts = depth / 4;
+  if (parts > 64) parts = 64;
+  return parts < 2 ? 1 : static_cast<int>(parts);
+}
+typedef hipError_t (*splitk_launcher)(const void*, const void*, void*, int, int, int, int, int, float*, hipStream_t);
+
 #define LEGO_GEMM_KERNELS_BIG_ONLY(DT)                                                                 \
   {{lego_gemm_##DT##_nn_launch, lego_gemm_##DT##_nt_launch, lego_gemm_##DT##_tn_launch,              \
     lego_gemm_##DT##_tt_launch},                                                                       \
@@ -357,6 +370,42 @@ int lego_hip_gemm_bf16_f16_ex(const void* a, const void* b, void* c, int M, int 
 {
   static const GemmKernels k = LEGO_GEMM_KERNELS(bf16h);
   return gemm_ex(k, 4, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
+}
+
+int lego_hip_gemm_workspace_bytes(int M, int N, int K, unsigned long long* bytes)
+{
+  if (bytes == nullptr || M <= 0 || N <= 0 || K <= 0) return kInvalid;
+  const int parts = splitk_parts(M, N, K, LEGO_GEMM_BK);
+  const unsigned long long tiles = static_cast<unsigned long long>((M + 127) / 128) * ((N + 127) / 128);
+  *bytes = parts > 1 ? parts * tiles * 128ull * 128ull * sizeof(float) : 0ull;
+  return 0;
+}
+
+int lego_hip_gemm_ex_ws(int element, const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
+                        int activation, void* workspace, unsigned long long workspace_bytes, void* stream)
+{
+#define LEGO_SPLITK(DT) {lego_gemm_##DT##_nn_t128x128_splitk_launch, lego_gemm_##DT##_nt_t128x128_splitk_launch, \
+                         lego_gemm_##DT##_tn_t128x128_splitk_launch, lego_gemm_##DT##_tt_t128x128_splitk_launch}
+  static const splitk_launcher f16[4] = LEGO_SPLITK(f16), bf16[4] = LEGO_SPLITK(bf16), bf16h[4] = LEGO_SPLITK(bf16h);
+#undef LEGO_SPLITK
+  if (element != 0 && element != 1 && element != 4) return kInvalid;
+  unsigned long long need = 0;
+  if (lego_hip_gemm_workspace_bytes(M, N, K, &need) != 0) return kInvalid;
+  // what the tiled kernels ask of shapes and bases (gemm_ex): anything else, and every product that gains nothing
+  // from parts, takes the plain entry point
+  const bool tiled = usable(a) && usable(b) && usable(c) && N % 8 == 0 && (trans_a ? M % 8 == 0 : K % 8 == 0) &&
+                     (!trans_b || K % 8 == 0);
+  if (need == 0 || !tiled || workspace == nullptr || workspace_bytes < need || !usable(workspace)) {
+    switch (element) {
+      case 0: return lego_hip_gemm_f16_ex(a, b, c, M, N, K, trans_a, trans_b, activation, stream);
+      case 1: return lego_hip_gemm_bf16_ex(a, b, c, M, N, K, trans_a, trans_b, activation, stream);
+      default: return lego_hip_gemm_bf16_f16_ex(a, b, c, M, N, K, trans_a, trans_b, activation, stream);
+    }
+  }
+  if (a == nullptr || b == nullptr || c == nullptr || (activation != 0 && activation != 1)) return kInvalid;
+  const splitk_launcher* by_layout = element == 0 ? f16 : element == 1 ? bf16 : bf16h;
+  return ok_or(by_layout[(trans_a ? 2 : 0) + (trans_b ? 1 : 0)](a, b, c, M, N, K, activation, splitk_parts(M, N, K, LEGO_GEMM_BK),
+                                                             static_cast<float*>(workspace), as_stream(stream)));
 }
 
 int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,

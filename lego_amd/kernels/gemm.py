@@ -290,6 +290,8 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
         c_out_row=code(c_out[0]), c_out_pair=code(c_out[1]),
         c_stage_load=code(tidy(4 * Cs_L[cr, 2 * cp], rng) - 4 * (cr % 2)),
         c_goff=code(tidy(C_L[pid_m, pid_n, wm * WM + cr, wn * WN + 8 * cp], rng)),
+        # the four columns that registers 4q..4q+3 of a lane hold of block (i, j): row and first column within the tile
+        c_goff_reg=code(tidy(C_L[pid_m, pid_n, idx("row"), idx("col")], {**rng, idx("row"): (0, bm), idx("col"): (0, bn)})),
         xcd_pid=code(tidy(xcd_remap(per_xcd, wg), {wg: (0, per_xcd * XCDS)})), CUS=CUS,
         pid_m=code(pm_e), pid_n=code(pn_e),
     )
@@ -316,7 +318,7 @@ def split_order(split, wg):
 
 
 def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, trans_b=False, with_grouped=True,
-         dtype="f16", with_split=False):
+         dtype="f16", with_split=False, with_splitk=False):
     """One translation unit: the GEMM kernel of one operand layout and element type on ``bm x bn``
     tiles, with ``with_grouped`` the grouped kernel on the same tiles, and with ``with_split`` a
     second grouped kernel that gives the last tiles of its launch to two workgroups each, as
@@ -325,7 +327,7 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
     params = _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped, dtype)
     ns = f"t{bm}x{bn}"
     tiles = [dict(ns=ns, text=template("gemm_tile.hip.j2").render(**params))]
-    params.update(main_ns=ns, with_split=with_split)
+    params.update(main_ns=ns, with_split=with_split, with_splitk=with_splitk)
     if with_split:
         assert with_grouped
         half = _tile_params(bm // 2, bn, bk, waves, max_group_m, trans_a, trans_b, True, dtype)
@@ -346,6 +348,8 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
     launchers = [f"lego_gemm_{dtype}_{variant}{tag}_launch"] + ([f"lego_grouped_gemm_f16{tag}_launch"] if with_grouped else [])
     if with_split:
         launchers.append(f"lego_grouped_gemm_f16{tag}_split_launch")
+    if with_splitk:
+        launchers.append(f"lego_gemm_{dtype}_{variant}{tag}_splitk_launch")
     return Emitted(f"gemm_{dtype}_{variant}{tag}.hip", text, launchers), meta
 
 

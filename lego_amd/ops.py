@@ -198,6 +198,15 @@ def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "", out_dtype=tor
         raise ValueError("out_dtype must be float16 or the operands' type")
     entry = "lego_hip_gemm_bf16_f16_ex" if (a.dtype, out_dtype) == (torch.bfloat16, torch.float16) else _GEMM_ENTRY[a.dtype]
     c = torch.empty((M, N), device=a.device, dtype=out_dtype)
+    # products of few tiles (a skinny operand, a long K) are split along K when there is room for the partial sums
+    need = ctypes.c_ulonglong(0)
+    runtime.call("lego_hip_gemm_workspace_bytes", M, N, K, ctypes.byref(need))
+    if need.value:
+        workspace = torch.empty(need.value // 4, dtype=torch.float32, device=a.device)
+        element = 0 if a.dtype == torch.float16 else 4 if out_dtype == torch.float16 else 1
+        runtime.call("lego_hip_gemm_ex_ws", element, _ptr(a_store), _ptr(b_store), _ptr(c), M, N, K, ta, tb,
+                     1 if activation else 0, _ptr(workspace), need, _stream())
+        return c
     runtime.call(entry, _ptr(a_store), _ptr(b_store), _ptr(c), M, N, K, ta, tb, 1 if activation else 0, _stream())
     return c
 

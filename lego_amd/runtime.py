@@ -37,6 +37,9 @@ SIGNATURES = {
                              _c_void_p],
     "lego_hip_gemm_bf16_f16_ex": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                   _c_void_p],
+    "lego_hip_gemm_workspace_bytes": [_c_int, _c_int, _c_int, ctypes.POINTER(ctypes.c_ulonglong)],
+    "lego_hip_gemm_ex_ws": [_c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                            _c_void_p, ctypes.c_ulonglong, _c_void_p],
     "lego_hip_gemm_fp8_ex": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                              _c_int, _c_void_p],
     "lego_hip_stencil_f3d_f32": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],

@@ -831,6 +831,81 @@ def test_gemm_offsets_beyond_32_bits(ops):
         assert _rel_err(c[rows].cpu(), ok.gemm(a[rows].cpu(), b.cpu())) <= 1e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(16, 2048, 2048), (1, 1024, 4096), (100, 264, 3000), (256, 256, 16384), (24, 4096, 520),
+                                   (2048, 16, 2048), (130, 130, 8200)])
+def test_gemm_split_along_k(ops, dtype, M, N, K):
+    """Products of few tiles get a workspace from the wrapper and are split along K: skinny operands, a long
+    K, ragged tiles and a ragged last k-tile (which falls to the last part).  Small integers (thinned out
+    so that every sum stays exact in 16 bits) in all four layouts, with and without the fused
+    activation; then random operands against the CPU oracle."""
+    import ctypes
+    from lego_amd import runtime
+    print(f"gemm split along k {dtype} {M}x{N}x{K}", flush=True)
+    need = ctypes.c_ulonglong(0)
+    runtime.call("lego_hip_gemm_workspace_bytes", M, N, K, ctypes.byref(need))
+    assert need.value > 0 and need.value % (128 * 128 * 4) == 0
+    g = _gen(81)
+    a = torch.randint(-2, 3, (M, K), generator=g).float()
+    b = torch.randint(-2, 3, (K, N), generator=g).float()
+    a = a * (torch.rand(M, K, generator=g) < min(1.0, 500.0 / K))      # about 500 non-zero terms of -4..4 per sum
+    want = a @ b
+    assert want.abs().max().item() <= 256          # exact in bfloat16 too
+    for ta in (False, True):
+        for tb in (False, True):
+            if ta and M % 8:
+                continue                # a transposed A of such an M is outside the tiled kernels
+            ad = a.to(dtype).cuda()
+            bd = b.to(dtype).cuda()
+            ad = ad.t().contiguous().t() if ta else ad
+            bd = bd.t().contiguous().t() if tb else bd
+            assert torch.equal(ops.matmul(ad, bd).cpu().float(), want), (ta, tb)
+            leaky = torch.where(want >= 0, want, 0.01 * want).half().float()
+            assert torch.equal(ops.matmul(ad, bd, activation="leaky_relu").cpu().float(), leaky), (ta, tb)
+    a = (torch.randn(M, K, generator=g) / math.sqrt(K)).to(dtype)
+    b = (torch.randn(K, N, generator=g) / math.sqrt(K)).to(dtype)
+    got = ops.matmul(a.cuda(), b.cuda()).cpu()
+    assert _rel_err(got, ok.gemm(a, b)) <= 1e-2
+
+
+def test_gemm_split_along_k_entry_point(ops):
+    """lego_hip_gemm_ex_ws through the C ABI: with the workspace it asks for it is bit-identical from call to
+    call (the parts are added in a fixed order) and within rounding of the plain entry point; with none, or a
+    short one, it IS the plain entry point; shapes with enough tiles ask for no workspace."""
+    import ctypes
+    from lego_amd import runtime
+    print("gemm split along k, entry point", flush=True)
+    M, N, K = 64, 1024, 8192
+    g = _gen(82)
+    a = (torch.randn(M, K, generator=g) / math.sqrt(K)).half().cuda()
+    b = (torch.randn(K, N, generator=g) / math.sqrt(K)).half().cuda()
+    need = ctypes.c_ulonglong(0)
+    runtime.call("lego_hip_gemm_workspace_bytes", M, N, K, ctypes.byref(need))
+    assert need.value > 0
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    plain = torch.empty(M, N, dtype=torch.half, device="cuda")
+    runtime.call("lego_hip_gemm_f16_ex", p(a), p(b), p(plain), M, N, K, 0, 0, 0, stream)
+    ws = torch.empty(need.value // 4, dtype=torch.float32, device="cuda")
+    outs = []
+    for fill in (0.0, float("nan")):            # whatever the workspace held
+        ws.fill_(fill)
+        c = torch.empty(M, N, dtype=torch.half, device="cuda")
+        runtime.call("lego_hip_gemm_ex_ws", 0, p(a), p(b), p(c), M, N, K, 0, 0, 0, p(ws), need, stream)
+        outs.append(c)
+    assert torch.equal(outs[0], outs[1])
+    assert (outs[0].float() - plain.float()).abs().max().item() <= 2e-3      # another summation order, one rounding
+    for workspace, size in ((None, 0), (p(ws), need.value - 1)):
+        c = torch.empty(M, N, dtype=torch.half, device="cuda")
+        runtime.call("lego_hip_gemm_ex_ws", 0, p(a), p(b), p(c), M, N, K, 0, 0, 0, workspace, ctypes.c_ulonglong(size), stream)
+        assert torch.equal(c, plain)
+    for shape in ((4096, 4096, 4096), (2048, 1024, 64), (128, 128, 256)):
+        runtime.call("lego_hip_gemm_workspace_bytes", *shape, ctypes.byref(need))
+        assert need.value == 0, shape
+    with pytest.raises(runtime.LegoHipError):
+        runtime.call("lego_hip_gemm_ex_ws", 2, p(a), p(b), p(plain), M, N, K, 0, 0, 0, p(ws), need, stream)   # 8-bit: no
+
+
 def test_gemm_rejects_bad_arguments(ops):
     with pytest.raises(ValueError):          # inner dimensions differ
         ops.matmul(torch.zeros(100, 64, device="cuda", dtype=torch.half),
