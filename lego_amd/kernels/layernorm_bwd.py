@@ -24,6 +24,11 @@ CONFIGS = ((256, 1), (256, 2), (256, 4), (512, 4))
 # that kernel only writes dx, and dw/db come from a second pass over dy and x by columns.
 LONG = (1024, 4)
 LONG_GROUPS = 64      # row slices of the column pass = rows of its partial buffers
+# rows of up to WAVE_MAX_N elements: a wavefront per row (1 or 2 vectors per lane), four rows per workgroup (with 4
+# vectors per lane a wave needs all 256 registers and 16384 x 2048 takes 57 us against 43)
+WAVE_VS = (1, 2)
+WAVE_MAX_N = 1024
+WAVE_GROUPS = 1024    # workgroups of those kernels = rows of their partial buffers
 
 
 def emit():
@@ -36,6 +41,7 @@ def emit():
     params = dict(
         banner=BANNER, CONFIGS=list(CONFIGS), MAX_GROUPS=MAX_GROUPS, LONG=LONG, LONG_GROUPS=LONG_GROUPS,
         KERNELS=[(th, v, True) for th, v in CONFIGS] + [LONG + (False,)],
+        WAVE_VS=WAVE_VS, WAVE_MAX_N=WAVE_MAX_N, WAVE_GROUPS=WAVE_GROUPS,
         MAX_N_ACC=max(th * v for th, v in CONFIGS) * 8,
         MAX_N_256=max(v for th, v in CONFIGS if th == 256) * 256 * 8,
         row_layout="OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])[step, wg]",
@@ -43,7 +49,7 @@ def emit():
         part_layout="OrderBy(Row(G, N)).TileBy([G, N/8], [1, 8])[wg, v, 0, :]",
         row=code(row_e),
         row_base=code(tidy(X[row, 0, 0, 0], {row: (0, M)})).replace("row", "static_cast<size_t>(row)"),
-        vecs={th: code(it * th + t) for th in sorted({th for th, _ in CONFIGS + (LONG,)})},
+        vecs={th: code(it * th + t) for th in sorted({64} | {th for th, _ in CONFIGS + (LONG,)})},
         vec_off=code(tidy(X[0, v, 0, 0], {v: (0, N / 8)})),
         vec_off4=code(tidy(OrderBy(Row(M, N)).TileBy([M, N / 4], [1, 4])[0, v, 0, 0], {v: (0, N / 4)})),
         stat_off=code(OrderBy(Row(M)).TileBy([M])[row,]),

@@ -310,7 +310,10 @@ def test_layernorm_backward_reference_test(ops):
 
 @pytest.mark.parametrize("M,N", [(1, 8), (3, 520), (700, 1024), (513, 2048), (64, 8192), (300, 8200), (129, 15872),
                                  (40, 16384), (5, 16392), (300, 24576), (70, 32768),
-                                 (3, 1), (5, 7), (17, 781), (130, 1000), (9, 4099), (4, 20001), (3, 32767)])
+                                 (3, 1), (5, 7), (17, 781), (130, 1000), (9, 4099), (4, 20001), (3, 32767),
+                                 # a wavefront per row, four rows per workgroup: fewer rows than waves, a last
+                                 # workgroup with one row, more rows than the 4096 teams of a full launch
+                                 (2, 512), (5, 256), (4101, 504), (9000, 1024), (6, 1016)])
 def test_layernorm_backward_matches_oracle(ops, M, N):
     print(f"layernorm backward {M}x{N}", flush=True)
     g = _gen(6)
