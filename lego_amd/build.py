@@ -45,12 +45,12 @@ TRANSPOSE = {
 ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f16", True, 8), ("f32", True, 1), ("f32", True, 4),
            ("f16", False, 1), ("f32", False, 1), ("f16", False, 4), ("f32", False, 4),
            ("f16", True, 16), ("f32", True, 16), ("f16", False, 16), ("f32", False, 16),
-           ("bf16", True, 1), ("bf16", True, 4), ("bf16", True, 16), ("bf16", False, 1), ("bf16", False, 4),
+           ("bf16", True, 1), ("bf16", True, 4), ("bf16", True, 8), ("bf16", True, 16), ("bf16", False, 1), ("bf16", False, 4),
            ("bf16", False, 16)]
 # (element type, lanes per row): teams of a part of a wave for rows of at most that many 16-byte vectors
 ROWWISE_SHORT = [(d, lanes) for d in ("f16", "bf16", "f32") for lanes in (16, 32)]
 # LayerNorm launches of many rows: this many workgroups that stage gamma and beta in LDS and walk the rows
-ROWWISE_STREAM_WGS = {("f16", True, 8): 512}
+ROWWISE_STREAM_WGS = {("f16", True, 8): 512, ("bf16", True, 8): 512}
 ROWWISE_DEFAULT_WAVES = 4
 ROWWISE_WIDE_TEAM_ABOVE_N, ROWWISE_WIDE_TEAM_FROM_M = 6144, 4096
 ROWWISE_MAX_N = rowwise.MAX_N
@@ -139,7 +139,7 @@ def collect():
           "// workgroup of 1024 lanes) hold the rows that four cannot",
           f"inline int lego_rowwise_default_wpr(int n) {{ return n <= 2048 ? 1 : n <= {rowwise.MAX_N_SMALL_TEAMS} ? "
           f"{ROWWISE_DEFAULT_WAVES} : {rowwise.LONG_ROW_WAVES}; }}",
-          "// fp16 rows of whole vectors: eight waves (a workgroup of 512 lanes, two to four vectors per lane) for long",
+          "// 16-bit rows of whole vectors: eight waves (a workgroup of 512 lanes, two to four vectors per lane) for long",
           "// rows of tall matrices, where they measure 3-5 % above four waves; fewer rows leave too few workgroups",
           f"inline int lego_rowwise_f16_wpr(int m, int n) {{ return n > {ROWWISE_WIDE_TEAM_ABOVE_N} && n <= "
           f"{rowwise.MAX_N_SMALL_TEAMS} && m >= {ROWWISE_WIDE_TEAM_FROM_M} ? 8 : lego_rowwise_default_wpr(n); }}", ""]

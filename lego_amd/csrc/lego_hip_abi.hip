@@ -191,6 +191,7 @@ int lego_hip_softmax_bf16(const void* x, void* y, int M, int N, void* stream)
     return ok_or((wpr == 16 ? lego_softmax_bf16s_w16_launch : wpr == 1 ? lego_softmax_bf16s_w1_launch
                                                                        : lego_softmax_bf16s_w4_launch)(x, y, M, N, as_stream(stream)));
   if (N <= 256) return ok_or((N <= 128 ? lego_softmax_bf16_l16_launch : lego_softmax_bf16_l32_launch)(x, y, M, N, as_stream(stream)));
+  if (lego_rowwise_f16_wpr(M, N) == 8) return ok_or(lego_softmax_bf16_w8_launch(x, y, M, N, as_stream(stream)));   // as fp16
   return ok_or((wpr == 16 ? lego_softmax_bf16_w16_launch : wpr == 1 ? lego_softmax_bf16_w1_launch
                                                                     : lego_softmax_bf16_w4_launch)(x, y, M, N, as_stream(stream)));
 }
@@ -208,6 +209,8 @@ int lego_hip_layernorm_fwd_bf16(const void* x, void* y, const void* w, const voi
   if (N <= 256)
     return ok_or((N <= 128 ? lego_layernorm_fwd_bf16_l16_launch : lego_layernorm_fwd_bf16_l32_launch)(
         x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+  if (lego_rowwise_f16_wpr(M, N) == 8)   // as fp16
+    return ok_or(lego_layernorm_fwd_bf16_w8_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
   return ok_or((wpr == 16 ? lego_layernorm_fwd_bf16_w16_launch : wpr == 1 ? lego_layernorm_fwd_bf16_w1_launch
                                                                           : lego_layernorm_fwd_bf16_w4_launch)(
       x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));

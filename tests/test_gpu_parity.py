@@ -389,7 +389,8 @@ def test_short_rows_share_a_wave(ops, dtype, M, N):
         _assert_layernorm_forward(y, x, w, b)
 
 
-@pytest.mark.parametrize("M,N", [(5, 8), (9, 781), (33, 2048), (64, 8192), (3, 8191), (4, 20000), (2, 32768), (2, 50257)])
+@pytest.mark.parametrize("M,N", [(5, 8), (9, 781), (33, 2048), (64, 8192), (3, 8191), (4, 20000), (2, 32768), (2, 50257),
+                                 (4100, 8200)])      # tall and long: teams of eight waves
 def test_softmax_bfloat16(ops, M, N):
     print(f"softmax bf16 {M}x{N}", flush=True)
     x = (2.0 * torch.randn(M, N, generator=_gen(30))).bfloat16()
@@ -400,7 +401,8 @@ def test_softmax_bfloat16(ops, M, N):
     assert (got.float() - want).abs().max().item() <= 2.0 ** -9 + 1e-6
 
 
-@pytest.mark.parametrize("M,N", [(5, 8), (9, 781), (33, 2048), (64, 8192), (3, 8191), (4, 20000), (2, 32768)])
+@pytest.mark.parametrize("M,N", [(5, 8), (9, 781), (33, 2048), (64, 8192), (3, 8191), (4, 20000), (2, 32768),
+                                 (4100, 8200)])      # tall and long: eight waves, gamma and beta staged in LDS
 def test_layernorm_bfloat16_forward_and_backward(ops, M, N):
     """bfloat16 tensors through the autograd wrapper, against fp32 autograd on the CPU."""
     from lego_amd.ops import lego_layer_norm
