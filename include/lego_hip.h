@@ -89,7 +89,7 @@ int lego_hip_layernorm_bwd_f32_workspace_bytes(int M, int N, unsigned long long*
 int lego_hip_layernorm_bwd_f32(const void* dy, const void* x, const void* w, const float* mean,
                                const float* rstd, void* dx, void* dw, void* db, void* workspace,
                                unsigned long long workspace_bytes, int M, int N, void* stream);
-/* ... and for bfloat16 tensors. */
+/* ... and for bfloat16 tensors, with the kernels and the workspace size of fp16. */
 int lego_hip_layernorm_bwd_bf16_workspace_bytes(int M, int N, unsigned long long* bytes);
 int lego_hip_layernorm_bwd_bf16(const void* dy, const void* x, const void* w, const float* mean,
                                 const float* rstd, void* dx, void* dw, void* db, void* workspace,
