@@ -342,6 +342,36 @@ def main():
                                                       frac_mfma=fl4 / ms8 / 1e9 / MFMA_FP8_PEAK_TFLOPS,
                                                       rel_err_vs_fp32=rel8, note="peak = 5.0 PFLOP/s dense fp8")
             del a8, b8, c8, ref8
+            # shapes off the tile grid: ragged in M and N (lane masks in scalar registers instead of edge tests), and
+            # a skinny product split along K with a workspace (bound by reading B once: GB/s of operand bytes)
+            mr = nr = 8184
+            cr = torch.empty(mr, nr, dtype=torch.float16, device="cuda")
+
+            br = b4[:, :nr].contiguous()      # rows 0..8183 of A are its first rows as they lie; B's columns need their own buffer
+
+            def gr2():
+                runtime.call("lego_hip_gemm_f16_ex", p(a4), p(br), p(cr), mr, nr, n4, 0, 0, 0, stream)
+            msr = timed(gr2, steps=max(5, K // 5), warmup=max(2, W // 5))
+            flr = 2.0 * mr * nr * n4
+            kernels["next_gemm_f16_8184x8184x8192_ragged"] = dict(ms=msr, tflops=flr / msr / 1e9,
+                                                                  frac_mfma=flr / msr / 1e9 / MFMA_F16_PEAK_TFLOPS)
+            del br, cr
+            ms_k = 16
+            a_s = a4[:ms_k].contiguous()
+            c_s = torch.empty(ms_k, n4, dtype=torch.float16, device="cuda")
+            need_s = ctypes.c_ulonglong(0)
+            runtime.call("lego_hip_gemm_workspace_bytes", ms_k, n4, n4, ctypes.byref(need_s))
+            ws_s = torch.empty(max(need_s.value, 16) // 4, device="cuda")
+
+            def gs():
+                runtime.call("lego_hip_gemm_ex_ws", 0, p(a_s), p(b4), p(c_s), ms_k, n4, n4, 0, 0, 0, p(ws_s), need_s, stream)
+            mss = timed(gs, steps=K, warmup=W)
+            lib_mss = timed(lambda: torch.matmul(a_s, b4, out=c_s), steps=K, warmup=W)
+            bytes_s = 2.0 * (ms_k * n4 + n4 * n4 + ms_k * n4)
+            kernels["next_gemm_f16_16x8192x8192_split_k"] = dict(ms=mss, gbs=bytes_s / mss / 1e6,
+                                                                 frac_hbm=bytes_s / mss / 1e6 / HBM_PEAK_GBS,
+                                                                 workspace_bytes=need_s.value, vendor_library_ms=lib_mss)
+            del a_s, c_s, ws_s
         del a4, b4, c4, ref
 
     # ---- C5: grouped fp16 GEMM, 8 problems -------------------------------------------------------------
