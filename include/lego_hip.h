@@ -146,7 +146,8 @@ int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, in
  * benchmarks/cuda/bricks_f3d.py:8-22 with bricks/main_tmp.cu:24-104, and bricks_laplasian.py:8-33
  * with bricks-laplace/main_tmp.cu:24-96).  bricks == 0: in and out are row-major; bricks != 0:
  * they are stored as contiguous 8 x 8 x 8 bricks, bricks in row-major order.  Points closer
- * than radius (1..3) to the boundary are not written.  n a multiple of 8, at most 1024.
+ * than radius (1..3; the laplacian, which the reference runs up to 4, 1..4) to the boundary are not written.
+ * n a multiple of 8, at most 1024.
  *   f3d:        out = in*c[r][r][r] + sum over |di|,|dj|,|dk| <= r of in[+di,+dj,+dk] * c[di+r][dj+r][dk+r],
  *               c an 8 x 8 x 8 array;
  *   laplacian:  out = in*c[0] + sum over a = 1..r of c[a] * (the six neighbours at distance a),

@@ -171,7 +171,8 @@ def collect():
     h += ["hipError_t lego_nw_i32_launch(const int*, int*, int, int, hipStream_t);",
           f"#define LEGO_NW_TILE {mnw['B']}", "",
           "hipError_t lego_stencil_f32_launch(const float*, float*, const float*, int, int, int, int, hipStream_t);",
-          f"#define LEGO_STENCIL_BRICK {mst['B']}", f"#define LEGO_STENCIL_MAX_RADIUS {mst['MAX_RADIUS']}", "",
+          f"#define LEGO_STENCIL_BRICK {mst['B']}", f"#define LEGO_STENCIL_MAX_RADIUS {mst['MAX_RADIUS']}",
+          f"#define LEGO_STENCIL_STAR_MAX_RADIUS {mst['STAR_MAX_RADIUS']}", "",
           "hipError_t lego_lud_f32_launch(float*, int, hipStream_t);", "hipError_t lego_lud_f32_plan(int, int*, int, int*);", f"#define LEGO_LUD_BLOCK {mlu['B']}", ""]
     return units, "\n".join(h)
 

@@ -435,7 +435,7 @@ namespace {
 int stencil(const float* in, float* out, const float* c, int n, int radius, int kind, int bricks, void* stream)
 {
   if (!usable(in) || !usable(out) || c == nullptr || in == out) return kInvalid;
-  if (n <= 0 || n % LEGO_STENCIL_BRICK || n > 1024 || radius < 1 || radius > LEGO_STENCIL_MAX_RADIUS || 2 * radius >= n)
+  if (n <= 0 || n % LEGO_STENCIL_BRICK || n > 1024 || radius < 1 || radius > (kind == 1 ? LEGO_STENCIL_STAR_MAX_RADIUS : LEGO_STENCIL_MAX_RADIUS) || 2 * radius >= n)
     return kInvalid;
   return ok_or(lego_stencil_f32_launch(in, out, c, n, radius, kind, bricks ? 1 : 0, as_stream(stream)));
 }

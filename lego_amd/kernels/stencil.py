@@ -30,6 +30,7 @@ from .common import BANNER, Emitted, code, idx, size, template, tidy
 
 B = 8
 MAX_RADIUS = 3        # the coefficient cube is 8 x 8 x 8: offsets -3..3 plus one unused plane
+STAR_MAX_RADIUS = 4   # the star stencil has radius + 1 coefficients; the reference runs it up to 4 (result/cuda/bricks-laplace.txt)
 WAVES = 4             # bricks per workgroup, dense stencil (its shell fills the 64 KiB of LDS at radius 3)
 STAR_WAVES = 8        # and star stencil: the more bricks in a row, the fewer row ends come from memory
 # words per row of the shell in LDS: 16 hold a row (3 + 8 + 3 points, 16-byte aligned), 20 spread the
@@ -86,7 +87,7 @@ def emit():
         shell_layout=f"OrderBy(Row(H, PLANE)).TileBy([H, PLANE])[hx, {ROW_WORDS}*hy + word]",
         shell_inv=shell_inv, shell_row=shell_row, ROW_WORDS=ROW_WORDS,
         PLANES={B + 2 * r: shell_plane(r) for r in range(1, MAX_RADIUS + 1)},
-        banner=BANNER, B=B, MAX_RADIUS=MAX_RADIUS, WAVES=WAVES, STAR_WAVES=STAR_WAVES,
+        banner=BANNER, B=B, MAX_RADIUS=MAX_RADIUS, STAR_MAX_RADIUS=STAR_MAX_RADIUS, WAVES=WAVES, STAR_WAVES=STAR_WAVES,
         row_layout=f"Row({B}, {B})",
         normal_layout=f"OrderBy(Row(N, N, N)).TileBy([N/{B}]*3, [{B}]*3)[x/{B}, y/{B}, z/{B}, x%{B}, y%{B}, z%{B}]",
         bricks_layout=f"OrderBy(Row(N/{B}, N/{B}, N/{B}), Row({B}, {B}, {B})).TileBy([N/{B}]*3, [{B}]*3)[x/{B}, ...]",
@@ -95,4 +96,4 @@ def emit():
         at_normal=at[0], at_bricks=at[1], coeff=code(coeff),
     )
     text = template("stencil.hip.j2").render(**params)
-    return Emitted("stencil_f32.hip", text, ["lego_stencil_f32_launch"]), dict(B=B, MAX_RADIUS=MAX_RADIUS)
+    return Emitted("stencil_f32.hip", text, ["lego_stencil_f32_launch"]), dict(B=B, MAX_RADIUS=MAX_RADIUS, STAR_MAX_RADIUS=STAR_MAX_RADIUS)

@@ -129,13 +129,14 @@ def test_gpu_f3d_matches_oracle(n, radius, bricks):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("bricks", [False, True])
-@pytest.mark.parametrize("n,radius", [(8, 1), (8, 3), (16, 1), (24, 3), (64, 2), (64, 3), (128, 1)])
+@pytest.mark.parametrize("n,radius", [(8, 1), (8, 3), (16, 1), (24, 3), (64, 2), (64, 3), (128, 1),
+                                      (16, 4), (40, 4), (64, 4)])      # radius 4: the reference's largest (result/cuda/bricks-laplace.txt)
 def test_gpu_laplacian_matches_oracle(n, radius, bricks):
     from lego_amd import ops
     print(f"laplacian n={n} radius={radius} bricks={bricks}", flush=True)
     g = torch.Generator().manual_seed(40 + n + radius)
     x = torch.rand(n, n, n, generator=g) * 2 - 1
-    c = torch.tensor([-6.0, 1.0, 0.5, 0.25])[:radius + 1].contiguous()
+    c = torch.tensor([-6.0, 1.0, 0.5, 0.25, 0.125])[:radius + 1].contiguous()
     want = torch.from_numpy(ok.stencil_laplacian(x.numpy(), c.numpy(), radius)).float()
     order = ok.bricks_order(n)
     xin = _to_bricks(x, order) if bricks else x
@@ -145,7 +146,7 @@ def test_gpu_laplacian_matches_oracle(n, radius, bricks):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("kind,radius", [("f3d", 1), ("f3d", 3), ("laplacian", 1), ("laplacian", 3)])
+@pytest.mark.parametrize("kind,radius", [("f3d", 1), ("f3d", 3), ("laplacian", 1), ("laplacian", 3), ("laplacian", 4)])
 def test_gpu_stencils_full_size_match_oracle_on_slabs(kind, radius):
     """The reference's size, 384^3, both storage orders, against the float64 oracle on three slabs of 16
     planes (the first, one across the middle of the brick grid, the last): the oracle of a slab widened
@@ -158,7 +159,7 @@ def test_gpu_stencils_full_size_match_oracle_on_slabs(kind, radius):
         c = torch.from_numpy(_coefficients(radius))
         call, oracle, tol = ops.stencil_f3d, ok.stencil_f3d, 2e-5 * (2 * radius + 1) ** 3
     else:
-        c = torch.tensor([-6.0, 1.0, 0.5, 0.25])[:radius + 1].contiguous()
+        c = torch.tensor([-6.0, 1.0, 0.5, 0.25, 0.125])[:radius + 1].contiguous()
         call, oracle, tol = ops.stencil_laplacian, ok.stencil_laplacian, 1e-5
     order = ok.bricks_order(n)
     rowmajor = call(x.cuda(), c.cuda(), radius, False).cpu()
