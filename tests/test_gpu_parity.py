@@ -656,6 +656,22 @@ def test_grouped_gemm_with_odd_problems(ops):
         assert ((c.cpu().float() - w.float()).abs() <= 2.0 ** -9 * w.float().abs() + 1e-3).all()
 
 
+def test_grouped_gemm_takes_up_to_64_problems(ops):
+    """The most problems one call takes (the kernels' argument block holds 64), all of different shape, many of a
+    single ragged tile; one more is refused."""
+    from lego_amd.runtime import LegoHipError
+    print("grouped gemm, 64 problems", flush=True)
+    g = _gen(45)
+    shapes = [(8 * (1 + (5 * i) % 37), 8 * (1 + (7 * i) % 29), 8 * (1 + (3 * i) % 23)) for i in range(64)]
+    A = [torch.randint(-2, 3, (m, k), generator=g).half() for m, n, k in shapes]
+    B = [torch.randint(-2, 3, (k, n), generator=g).half() for m, n, k in shapes]
+    got = ops.lego_group_gemm_fn([a.cuda() for a in A], [b.cuda() for b in B])
+    for a, b, c in zip(A, B, got):
+        assert torch.equal(c.cpu().float(), a.float() @ b.float())      # small integers: exact
+    with pytest.raises(LegoHipError):
+        ops.lego_group_gemm_fn([a.cuda() for a in A + A[:1]], [b.cuda() for b in B + B[:1]])
+
+
 def _grouped_call(entry, A, B, *extra):
     """Call a grouped entry point through the C ABI on device tensors; returns the results."""
     import ctypes
