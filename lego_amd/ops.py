@@ -24,14 +24,16 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _stream():
-    """The current stream's handle; asked for on every call, since the caller may switch streams."""
-    if _raw_stream is not None:      # a plain integer, without building a torch.cuda.Stream object
-        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    """The current stream's handle (an integer, or None for the null stream: what a ``c_void_p`` parameter takes);
+    asked for on every call, since the caller may switch streams."""
+    if _raw_stream is not None:      # without building a torch.cuda.Stream object
+        return _raw_stream(torch.cuda.current_device()) or None
+    return torch.cuda.current_stream().cuda_stream or None
 
 
 def _ptr(t):
-    return ctypes.c_void_p(t.data_ptr())
+    """The tensor's address as an integer (None for an empty tensor's null pointer): a ``c_void_p`` parameter."""
+    return t.data_ptr() or None
 
 
 def _check(t, dtype, name, ndim=2):
@@ -82,7 +84,7 @@ def layer_norm_fwd(x, weight, bias, eps=1e-5, waves_per_row: int | None = None):
     """LayerNorm forward over the last dimension; returns ``(y, mean, rstd)``."""
     if x.dtype not in _ROW_TAG:
         raise ValueError("x must be float16, bfloat16 or float32")
-    x_arg = x.reshape(-1, x.shape[-1])
+    x_arg = x if x.dim() == 2 else x.reshape(-1, x.shape[-1])      # every torch call here costs a microsecond
     _check(x_arg, x.dtype, "x")
     M, N = x_arg.shape
     _check(weight, x.dtype, "weight", ndim=1)
@@ -102,7 +104,7 @@ def layer_norm_fwd(x, weight, bias, eps=1e-5, waves_per_row: int | None = None):
         raise ValueError("waves_per_row is a tuning knob of the fp16 kernels")
     else:
         runtime.call("lego_hip_layernorm_fwd_f16_wpr", *args, waves_per_row, _stream())
-    return y.view(x.shape), mean, rstd
+    return (y if x.dim() == 2 else y.view(x.shape)), mean, rstd
 
 
 def layer_norm_bwd(dy, x, weight, mean, rstd):
@@ -110,8 +112,8 @@ def layer_norm_bwd(dy, x, weight, mean, rstd):
     if x.dtype not in _ROW_TAG:
         raise ValueError("x must be float16, bfloat16 or float32")
     tag = _ROW_TAG[x.dtype]
-    x_arg = x.reshape(-1, x.shape[-1])
-    dy_arg = dy.reshape(-1, dy.shape[-1]).contiguous()
+    x_arg = x if x.dim() == 2 else x.reshape(-1, x.shape[-1])
+    dy_arg = dy if dy.dim() == 2 and dy.is_contiguous() else dy.reshape(-1, dy.shape[-1]).contiguous()
     _check(x_arg, x.dtype, "x")
     _check(dy_arg, x.dtype, "dy")
     _check(weight, x.dtype, "weight", ndim=1)
@@ -132,7 +134,7 @@ def layer_norm_bwd(dy, x, weight, mean, rstd):
     db = torch.empty((N,), dtype=weight.dtype, device=x.device)
     runtime.call(f"lego_hip_layernorm_bwd_{tag}", _ptr(dy_arg), _ptr(x_arg), _ptr(weight), _ptr(mean), _ptr(rstd),
                  _ptr(dx), _ptr(dw), _ptr(db), _ptr(workspace), need, M, N, _stream())
-    return dx.view(x.shape), dw, db
+    return (dx if x.dim() == 2 else dx.view(x.shape)), dw, db
 
 
 class LEGOLayerNorm(torch.autograd.Function):

@@ -96,8 +96,14 @@ def load_library(path=None):
     return lib
 
 
+_entry_points = {}
+
+
 def call(entry, *args):
     """Call one entry point and raise ``LegoHipError`` on a non-zero return."""
-    code = getattr(load_library(), entry)(*args)
+    fn = _entry_points.get(entry)
+    if fn is None:      # looked up once: the wrappers sit in front of kernels of a few microseconds
+        fn = _entry_points[entry] = getattr(load_library(), entry)
+    code = fn(*args)
     if code != 0:
         raise LegoHipError(entry, code)
