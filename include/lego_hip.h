@@ -83,8 +83,9 @@ int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, con
 int lego_hip_layernorm_bwd_f16_noalloc(const void* dy, const void* x, const void* w, const float* mean,
                                        const float* rstd, void* dx, void* dw, void* db, int M, int N, void* stream);
 
-/* The same for fp32 tensors (the reference's kernels take the tensors' own type, layernorm.py:372-405);
- * every shape takes the two passes; the workspace has its own size. */
+/* The same for fp32 tensors (the reference's kernels take the tensors' own type, layernorm.py:372-405): the
+ * kernels of fp16 for rows in whole groups of eight elements, two passes otherwise; the workspace has its
+ * own size. */
 int lego_hip_layernorm_bwd_f32_workspace_bytes(int M, int N, unsigned long long* bytes);
 int lego_hip_layernorm_bwd_f32(const void* dy, const void* x, const void* w, const float* mean,
                                const float* rstd, void* dx, void* dw, void* db, void* workspace,

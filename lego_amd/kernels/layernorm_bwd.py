@@ -42,8 +42,8 @@ def emit():
         banner=BANNER, CONFIGS=list(CONFIGS), MAX_GROUPS=MAX_GROUPS, LONG=LONG, LONG_GROUPS=LONG_GROUPS,
         KERNELS=[(th, v, True) for th, v in CONFIGS] + [LONG + (False,)],
         WAVE_VS=WAVE_VS, WAVE_MAX_N=WAVE_MAX_N, WAVE_GROUPS=WAVE_GROUPS,
-        # the two 16-bit element types take the same kernels: (type, tag, vector type)
-        ELTS16=[("_Float16", "f16", "half8"), ("__bf16", "bf16", "bhalf8")],
+        # every element type takes the same kernels, eight elements per lane and step: (type, tag, vector type)
+        ELTS=[("_Float16", "f16", "half8"), ("__bf16", "bf16", "bhalf8"), ("float", "f32", "float8v")],
         MAX_N_ACC=max(th * v for th, v in CONFIGS) * 8,
         MAX_N_256=max(v for th, v in CONFIGS if th == 256) * 256 * 8,
         row_layout="OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])[step, wg]",

@@ -345,7 +345,10 @@ def test_layernorm_backward_rejects_foreign_statistics(ops):
         ops.layer_norm_bwd(torch.zeros(4, 32, dtype=torch.half, device="cuda"), x, w, good, good)
 
 
-@pytest.mark.parametrize("M,N", [(1, 4), (7, 5), (300, 1000), (129, 4096), (33, 4099), (40, 16384)])
+@pytest.mark.parametrize("M,N", [(1, 4), (7, 5), (300, 1000), (129, 4096), (33, 4099), (40, 16384),
+                                 # rows in whole groups of eight take the fused kernels: a wavefront per row (512, 1016),
+                                 # 256 lanes with 1, 2 and 4 groups per lane, 512 lanes; 1004 is in whole vectors only
+                                 (4101, 512), (70, 1016), (600, 2048), (50, 3000), (513, 8192), (9, 12288), (30, 1004)])
 def test_layernorm_backward_fp32(ops, M, N):
     """fp32 tensors through the autograd wrapper, against fp64 autograd on the CPU."""
     from lego_amd.ops import lego_layer_norm
