@@ -72,7 +72,7 @@ def emit(waves_per_row=1, dtype="f16", vectorised=True, seq_max_wpr=4, prefetch_
         VPTS=[1] if team_lanes else [vp for vp in VPTS if vp * EPV <= 128 and lo < vp * TEAM * EPV <= hi],
         dtype=dtype, elt=elt, EPV=EPV, ESIZE=esize, RAGGED=not vectorised, tag=tag,
         SEQ_MAX_WPR=seq_max_wpr, PREFETCH_MAX_WPR=prefetch_max_wpr,
-        STREAM=vectorised and RPW == 1 and WPR < LONG_ROW_WAVES and stream_wgs > 0, STREAM_WGS=stream_wgs,
+        STREAM=vectorised and RPW == 1 and stream_wgs > 0, STREAM_WGS=stream_wgs,
         stream_layout="OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])[step, wg]", stream_row=code(stream_row),
         row_layout=f"OrderBy(Row(NWG, {RPW})).TileBy([NWG], [{RPW}])[wg, team]",
         lane_layout=f"OrderBy(Row({RPW}, {TEAM})).TileBy([{RPW}, {TEAM}]).inv(t); vector = it*{TEAM} + lane",

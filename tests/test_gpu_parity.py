@@ -249,8 +249,9 @@ def test_layernorm_fp32_long_rows_through_the_c_abi(ops, N):
 
 @pytest.mark.parametrize("wpr", [None, 1, 2, 4, 8])
 # 1151 and 4100 rows with eight waves: workgroups that stage gamma and beta in LDS and walk two to nine rows each
+# 600 and 515 rows of more than 16384 elements: the same walk with sixteen waves, one row across 1024 lanes
 @pytest.mark.parametrize("M,N", [(7, 8), (33, 520), (64, 1024), (129, 4096), (1151, 8192), (3, 16384), (4100, 8200),
-                                 (1030, 16384)])
+                                 (1030, 16384), (600, 32768), (515, 20488), (511, 32768)])
 def test_layernorm_matches_oracle(ops, M, N, wpr):
     print(f"layernorm {M}x{N} wpr={wpr}", flush=True)
     if wpr is not None and N > min(8192 * wpr, 16384):
@@ -405,7 +406,7 @@ def test_softmax_bfloat16(ops, M, N):
 
 
 @pytest.mark.parametrize("M,N", [(5, 8), (9, 781), (33, 2048), (64, 8192), (3, 8191), (4, 20000), (2, 32768),
-                                 (4100, 8200)])      # tall and long: eight waves, gamma and beta staged in LDS
+                                 (4100, 8200), (530, 24576)])   # tall and long: gamma and beta staged in LDS
 def test_layernorm_bfloat16_forward_and_backward(ops, M, N):
     """bfloat16 tensors through the autograd wrapper, against fp32 autograd on the CPU."""
     from lego_amd.ops import lego_layer_norm
