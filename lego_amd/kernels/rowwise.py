@@ -66,13 +66,19 @@ def emit(waves_per_row=1, dtype="f16", vectorised=True, seq_max_wpr=4, prefetch_
     # Row(STEPS, G)[step, wg]
     G, STEPS, step = size("G"), size("STEPS"), idx("step")
     stream_row = tidy(OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])[step, wg], {step: (0, STEPS), wg: (0, G)})
+    # the same walk with several teams per workgroup (rows of any length): Row(STEPS, G, RPW)[step, wg, team]
+    team_rows = OrderBy(Row(STEPS, G, RPW)).TileBy([STEPS], [G], [RPW])
+    stream_team_row = tidy(team_rows[step, wg, team], {step: (0, STEPS), wg: (0, G), team: (0, RPW)})
+    stream_team0_row = tidy(team_rows[step, wg, 0], {step: (0, STEPS), wg: (0, G)})
 
     params = dict(
         banner=BANNER, WPR=WPR, TEAM=TEAM, RPW=RPW, THREADS=threads, WTAG=wtag, SHUFFLE=min(TEAM, 64),
         VPTS=[1] if team_lanes else [vp for vp in VPTS if vp * EPV <= 128 and lo < vp * TEAM * EPV <= hi],
         dtype=dtype, elt=elt, EPV=EPV, ESIZE=esize, RAGGED=not vectorised, tag=tag,
         SEQ_MAX_WPR=seq_max_wpr, PREFETCH_MAX_WPR=prefetch_max_wpr,
-        STREAM=vectorised and RPW == 1 and stream_wgs > 0, STREAM_WGS=stream_wgs,
+        STREAM=stream_wgs > 0 and (RPW == 1 or not vectorised), STREAM_WGS=stream_wgs,
+        stream_team_layout=f"OrderBy(Row(STEPS, G, {RPW})).TileBy([STEPS], [G], [{RPW}])[step, wg, team]",
+        stream_team_row=code(stream_team_row), stream_team0_row=code(stream_team0_row),
         stream_layout="OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])[step, wg]", stream_row=code(stream_row),
         row_layout=f"OrderBy(Row(NWG, {RPW})).TileBy([NWG], [{RPW}])[wg, team]",
         lane_layout=f"OrderBy(Row({RPW}, {TEAM})).TileBy([{RPW}, {TEAM}]).inv(t); vector = it*{TEAM} + lane",

@@ -189,7 +189,10 @@ def test_softmax_reference_test_shape_fp32(ops):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("M,N", [(5, 1), (9, 3), (17, 781), (4, 1000), (3, 4099), (2, 16383), (6, 2048), (3, 16384),
-                                 (3, 16392), (2, 20001), (5, 32767), (4, 32768)])
+                                 (3, 16392), (2, 20001), (5, 32767), (4, 32768),
+                                 # tall and ragged: teams walk rows that start alike, the next row's loads in flight
+                                 (8300, 781), (8195, 250), (8200, 1001), (2050, 4099), (2049, 8191), (2300, 2050),
+                                 (1030, 12001), (1100, 16383), (515, 20001), (600, 32767)])
 def test_softmax_ragged_and_fp32(ops, dtype, M, N):
     print(f"softmax {dtype} {M}x{N}", flush=True)
     x = (2.0 * torch.randn(M, N, generator=_gen(2))).to(dtype)
@@ -200,7 +203,10 @@ def test_softmax_ragged_and_fp32(ops, dtype, M, N):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("M,N", [(5, 1), (9, 3), (17, 781), (3, 4099), (6, 2048), (3, 16384), (3, 16392), (2, 20001),
-                                 (4, 32768)])
+                                 (4, 32768),
+                                 # tall and ragged: teams walk rows that start alike, gamma and beta shifted into LDS
+                                 (8300, 781), (8195, 250), (8200, 1001), (2050, 4099), (2049, 8191), (2300, 2050),
+                                 (515, 20001), (600, 32767), (1030, 12001), (1100, 16383), (4100, 3001)])
 def test_layernorm_ragged_and_fp32(ops, dtype, M, N):
     print(f"layernorm {dtype} {M}x{N}", flush=True)
     if N * torch.empty((), dtype=dtype).element_size() > 65536:
