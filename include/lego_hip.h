@@ -64,8 +64,9 @@ int lego_hip_layernorm_fwd_bf16(const void* x, void* y, const void* w, const voi
  * partial buffers become one fp32 workspace the caller provides (the reference's wrapper
  * allocates its buffers with torch as well): ask for its size first, any 16-byte aligned
  * device buffer of at least that many bytes will do; its contents need no initialisation.
- * Any N up to 32768 (the reference's fp16 limit); rows above 16384 elements and rows whose length
- * is not a multiple of 8 are read twice (dx by rows, then dw/db by columns). */
+ * Any N up to 32768 (the reference's fp16 limit); rows above 16384 elements are read twice (dx by
+ * rows, then dw/db by columns).  Rows of a length that is not a multiple of 8 are split at their 16-byte
+ * boundaries, which fall on the same columns in dy, x and dx (16-byte aligned buffers of one shape). */
 int lego_hip_layernorm_bwd_workspace_bytes(int M, int N, unsigned long long* bytes);
 int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, const float* mean,
                                const float* rstd, void* dx, void* dw, void* db, void* workspace,
@@ -84,8 +85,7 @@ int lego_hip_layernorm_bwd_f16_noalloc(const void* dy, const void* x, const void
                                        const float* rstd, void* dx, void* dw, void* db, int M, int N, void* stream);
 
 /* The same for fp32 tensors (the reference's kernels take the tensors' own type, layernorm.py:372-405): the
- * kernels of fp16 for rows in whole groups of eight elements, two passes otherwise; the workspace has its
- * own size. */
+ * kernels of fp16 for rows of up to 16384 elements, two passes above; the workspace has its own size. */
 int lego_hip_layernorm_bwd_f32_workspace_bytes(int M, int N, unsigned long long* bytes);
 int lego_hip_layernorm_bwd_f32(const void* dy, const void* x, const void* w, const float* mean,
                                const float* rstd, void* dx, void* dw, void* db, void* workspace,

@@ -18,10 +18,14 @@ from .common import BANNER, Emitted, code, idx, size, template, tidy
 MAX_GROUPS = 512      # workgroups of stage 1 = rows of the partial buffers
 # (lanes per row, 16-byte vectors per lane): rows of up to 2048, 4096, 8192 and 16384 elements; the
 # longest rows take 512 lanes so that a lane's partial sums still fit its registers
-CONFIGS = ((256, 1), (256, 2), (256, 4), (512, 4))
+CONFIGS = ((256, 1), (256, 2), (512, 2), (512, 4))
 # Longer rows (the reference takes fp16 rows of up to 32768 elements, layernorm_triton.py:398-401):
 # 1024 lanes per row leave a lane 128 registers, too few for its partial sums next to the row, so
 # that kernel only writes dx, and dw/db come from a second pass over dy and x by columns.
+# Rows of any length keep a few more values per lane (their head and tail elements): with four vectors per lane 256
+# lanes pass 256 registers and only one workgroup stays on a CU, so rows of 4097-8192 elements take 512 lanes
+# with two vectors each and the next row's loads in flight
+RAGGED_CONFIGS = ((256, 1), (256, 2), (512, 2), (512, 4))
 LONG = (1024, 4)
 LONG_GROUPS = 64      # row slices of the column pass = rows of its partial buffers
 # rows of up to WAVE_MAX_N elements: a wavefront per row (1 or 2 vectors per lane), four rows per workgroup (with 4
@@ -40,7 +44,10 @@ def emit():
     P = OrderBy(Row(G, N)).TileBy([G, N / 8], [1, 8])
     params = dict(
         banner=BANNER, CONFIGS=list(CONFIGS), MAX_GROUPS=MAX_GROUPS, LONG=LONG, LONG_GROUPS=LONG_GROUPS,
-        KERNELS=[(th, v, True) for th, v in CONFIGS] + [LONG + (False,)],
+        # (lanes, vectors per lane, keeps partial sums, rows of any length)
+        KERNELS=[(th, v, True, False) for th, v in CONFIGS] + [(th, v, True, True) for th, v in RAGGED_CONFIGS]
+        + [LONG + (False, False)],
+        RAGGED_CONFIGS=list(RAGGED_CONFIGS), RAGGED_MAX_N_256=max(v for th, v in RAGGED_CONFIGS if th == 256) * 256 * 8,
         WAVE_VS=WAVE_VS, WAVE_MAX_N=WAVE_MAX_N, WAVE_GROUPS=WAVE_GROUPS,
         # every element type takes the same kernels, eight elements per lane and step: (type, tag, vector type)
         ELTS=[("_Float16", "f16", "half8"), ("__bf16", "bf16", "bhalf8"), ("float", "f32", "float8v")],

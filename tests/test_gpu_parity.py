@@ -320,7 +320,11 @@ def test_layernorm_backward_reference_test(ops):
                                  (3, 1), (5, 7), (17, 781), (130, 1000), (9, 4099), (4, 20001), (3, 32767),
                                  # a wavefront per row, four rows per workgroup: fewer rows than waves, a last
                                  # workgroup with one row, more rows than the 4096 teams of a full launch
-                                 (2, 512), (5, 256), (4101, 504), (9000, 1024), (6, 1016)])
+                                 (2, 512), (5, 256), (4101, 504), (9000, 1024), (6, 1016),
+                                 # rows of any length, more rows than workgroups: a workgroup's rows start alike and
+                                 # split into head, vectors and tail at the same columns
+                                 (1100, 781), (700, 1001), (1030, 2050), (600, 4099), (530, 8191), (300, 12001),
+                                 (515, 16383), (520, 250), (1100, 33), (513, 7)])
 def test_layernorm_backward_matches_oracle(ops, M, N):
     print(f"layernorm backward {M}x{N}", flush=True)
     g = _gen(6)
@@ -355,7 +359,9 @@ def test_layernorm_backward_rejects_foreign_statistics(ops):
 @pytest.mark.parametrize("M,N", [(1, 4), (7, 5), (300, 1000), (129, 4096), (33, 4099), (40, 16384),
                                  # rows in whole groups of eight take the fused kernels: a wavefront per row (512, 1016),
                                  # 256 lanes with 1, 2 and 4 groups per lane, 512 lanes; 1004 is in whole vectors only
-                                 (4101, 512), (70, 1016), (600, 2048), (50, 3000), (513, 8192), (9, 12288), (30, 1004)])
+                                 (4101, 512), (70, 1016), (600, 2048), (50, 3000), (513, 8192), (9, 12288), (30, 1004),
+                                 # rows of any length through the same kernels
+                                 (1100, 781), (600, 4099), (530, 8190), (300, 12001), (1030, 1003), (515, 16381)])
 def test_layernorm_backward_fp32(ops, M, N):
     """fp32 tensors through the autograd wrapper, against fp64 autograd on the CPU."""
     from lego_amd.ops import lego_layer_norm
@@ -412,7 +418,8 @@ def test_softmax_bfloat16(ops, M, N):
 
 
 @pytest.mark.parametrize("M,N", [(5, 8), (9, 781), (33, 2048), (64, 8192), (3, 8191), (4, 20000), (2, 32768),
-                                 (4100, 8200), (530, 24576)])   # tall and long: gamma and beta staged in LDS
+                                 (4100, 8200), (530, 24576),    # tall and long: gamma and beta staged in LDS
+                                 (1100, 781), (530, 8191), (260, 16383)])
 def test_layernorm_bfloat16_forward_and_backward(ops, M, N):
     """bfloat16 tensors through the autograd wrapper, against fp32 autograd on the CPU."""
     from lego_amd.ops import lego_layer_norm
