@@ -32,13 +32,15 @@ TRANSPOSE = {
             dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 32, 8), max_bytes=256 << 20),
             dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag"),
             dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag"),
-            dict(dtype="f32", tile=(32, 32), group=(2, 4), order="diag", edge=True)],
+            dict(dtype="f32", tile=(32, 32), group=(2, 4), order="diag", edge=True),
+            dict(dtype="f32", tile=(32, 32), group=(2, 4), order="diag", edge=True, ragged=True)],
     "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 128, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 64, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 32, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag"),
             dict(dtype="f16", tile=(64, 64), group=(1, 1), order="diag"),
-            dict(dtype="f16", tile=(64, 64), group=(2, 2), order="diag", edge=True)],
+            dict(dtype="f16", tile=(64, 64), group=(2, 2), order="diag", edge=True),
+            dict(dtype="f16", tile=(64, 64), group=(2, 2), order="diag", edge=True, ragged=True)],
 }
 # (element type, vectorised, waves per row): 16-byte accesses need N % (16/size) == 0; the
 # element-per-access kernels ("s") take any N
@@ -78,6 +80,10 @@ def collect():
             if cfg.get("edge"):
                 vec = 4 if dtype == "f32" else 8
                 meta["row_multiple"] = meta["col_multiple"] = vec
+            if cfg.get("ragged"):     # any shape with at least one whole vector per row of both matrices
+                meta["row_multiple"] = meta["col_multiple"] = 1
+                meta["min_side"] = vec
+                meta["min_elements"] = 256 * meta["SR"] * meta["SC"]     # a macro tile per CU; smaller matrices take 64x64 tiles
             unit.filename = meta["kernel"].replace("lego_", "", 1) + ".hip"
             units.append(unit)
             tmeta.setdefault(dtype, []).append(meta)
@@ -116,12 +122,14 @@ def collect():
     for dtype, metas in tmeta.items():
         for m in metas:
             h.append(f"hipError_t {m['kernel']}_launch(const void*, void*, int, int, hipStream_t);")
-        h += [f"// picks the first tiling that divides the shape, else the one-element-per-access kernel",
+        h += [f"// picks the first tiling that divides the shape; any other shape takes the same tiling with vectors at any element and edge tests, a small matrix the one-element-per-access kernel (64x64 tiles)",
               f"inline hipError_t lego_transpose_{dtype}_dispatch(const void* in, void* out, int rows, int cols, "
               "hipStream_t stream) {"]
         for m in metas:
             fits = "" if m["max_bytes"] is None else \
                 f" && 2ull * rows * cols * {4 if dtype == 'f32' else 2} <= {m['max_bytes']}ull"
+            if m.get("min_side"):
+                fits += f" && rows >= {m['min_side']} && cols >= {m['min_side']} && 1ull * rows * cols >= {m['min_elements']}ull"
             h.append(f"  if (rows % {m['row_multiple']} == 0 && cols % {m['col_multiple']} == 0{fits}) "
                      f"return {m['kernel']}_launch(in, out, rows, cols, stream);")
         h += [f"  return lego_transpose_any_launch(in, out, rows, cols, {4 if dtype == 'f32' else 2}, stream);", "}", ""]

@@ -79,16 +79,29 @@ def test_transpose_moves_bits_of_any_2_or_4_byte_type(ops, dtype):
                                              (torch.float16, 8, 8), (torch.float16, 72, 264), (torch.float16, 1000, 520),
                                              (torch.float16, 4104, 1096), (torch.float16, 64, 8), (torch.float16, 8, 1024),
                                              (torch.float32, 4, 4), (torch.float32, 36, 260), (torch.float32, 1004, 516),
-                                             (torch.float32, 2052, 4100)])
+                                             (torch.float32, 2052, 4100),
+                                             # rows that start at any element: vectors at their own alignment, the ones
+                                             # that an edge cuts element by element
+                                             (torch.float16, 9, 9), (torch.float16, 1001, 999), (torch.float16, 130, 257),
+                                             (torch.float16, 2055, 1031), (torch.float16, 15, 4099), (torch.float16, 4099, 15),
+                                             (torch.float16, 1000, 777), (torch.float16, 777, 1000), (torch.float16, 7, 300),
+                                             (torch.float32, 5, 7), (torch.float32, 1001, 999), (torch.float32, 130, 257),
+                                             (torch.float32, 2051, 1033), (torch.float32, 516, 1001), (torch.float32, 1001, 516),
+                                             # ... from a macro tile per CU on (smaller matrices take the 64x64 tiles)
+                                             (torch.float16, 2055, 2061), (torch.float16, 15, 300001), (torch.float16, 300001, 15),
+                                             (torch.float16, 4100, 1031), (torch.float16, 1031, 4100),
+                                             (torch.float32, 1449, 1451), (torch.float32, 5, 500001), (torch.float32, 500001, 5),
+                                             (torch.float32, 2052, 1031)])
 def test_transpose_of_any_shape(ops, dtype, rows, cols):
     """Shapes no tiling divides: in whole 16-byte vectors both ways they take the wide tile with edge
-    tests, otherwise the one-element-per-access kernel."""
+    tests, otherwise the same tile with vectors at any element, and the one-element-per-access kernel when a
+    side is shorter than a vector."""
     print(f"transpose (any shape) {dtype} {rows}x{cols}", flush=True)
     x = (torch.rand(rows, cols, generator=_gen(4)) * 2 - 1).to(dtype)
     want = ok.transpose(x, 1, 1)
     assert torch.equal(want, x.t().contiguous())
-    buf = torch.full((rows * cols + 1024,), 7.0, dtype=dtype, device="cuda")
-    out = buf[:rows * cols].view(cols, rows)
+    buf = torch.full((rows * cols + 2048,), 7.0, dtype=dtype, device="cuda")
+    out = buf[1024:1024 + rows * cols].view(cols, rows)
     from lego_amd import runtime
     import ctypes
     xd = x.cuda()
@@ -96,7 +109,7 @@ def test_transpose_of_any_shape(ops, dtype, rows, cols):
                  ctypes.c_void_p(xd.data_ptr()), ctypes.c_void_p(out.data_ptr()), rows, cols, None)
     torch.cuda.synchronize()
     assert torch.equal(out.cpu(), want)
-    assert (buf[rows * cols:] == 7.0).all()       # nothing past the matrix was written
+    assert (buf[:1024] == 7.0).all() and (buf[1024 + rows * cols:] == 7.0).all()       # nothing outside the matrix was written
 
 
 def test_transpose_offsets_beyond_32_bits(ops):
