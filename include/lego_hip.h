@@ -128,11 +128,13 @@ int lego_hip_gemm_bf16_f16_ex(const void* a, const void* b, void* c, int M, int 
  * sums.  A product of few tiles -- a skinny operand (16 x 8192 x 8192), a long K (256 x 256 x 65536) -- leaves most
  * CUs idle with one workgroup per tile and cannot pull its operands through the chip; with a workspace the k-tiles
  * of every tile are dealt to several workgroups, which leave fp32 sums there, and a second kernel adds them in a
- * fixed order (deterministic), applies the activation and stores C.  lego_hip_gemm_workspace_bytes gives the size
- * the call uses for a shape (0: it gains nothing from parts).  The workspace is scratch: 16-byte aligned device
- * memory, contents undefined on entry and exit, not to be shared by calls that may overlap.  With a null or short
- * workspace, or a shape outside the tiled kernels, the call is lego_hip_gemm_*_ex.  No counterpart in the
- * reference, whose matmul has one program per tile (matmul_sympy.py:57-65). */
+ * fixed order (deterministic), applies the activation and stores C.  A product with N or K that is not a multiple
+ * of 8 (operand rows that are not whole 16-byte chunks) runs on zero-padded copies of A, B and C in the workspace
+ * instead of the one-element-per-access kernel, about ten times as fast; operands may then start at any element.
+ * lego_hip_gemm_workspace_bytes gives the size the call uses for a shape (0: it gains nothing from a workspace).
+ * The workspace is scratch: 16-byte aligned device memory, contents undefined on entry and exit, not to be shared
+ * by calls that may overlap.  With a null or short workspace the call is lego_hip_gemm_*_ex.  No counterpart in
+ * the reference, whose matmul has one program per tile (matmul_sympy.py:57-65). */
 int lego_hip_gemm_workspace_bytes(int M, int N, int K, unsigned long long* bytes);
 int lego_hip_gemm_ex_ws(int element, const void* a, const void* b, void* c, int M, int N, int K, int trans_a,
                         int trans_b, int activation, void* workspace, unsigned long long workspace_bytes,

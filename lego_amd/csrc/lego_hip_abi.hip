@@ -41,6 +41,72 @@ __global__ void __launch_bounds__(256) lego_copy16_stream_kernel(const u32x4* __
   for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(v[u], out + base + u * 256);
 }
 
+typedef unsigned u32x4w __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4w_any __attribute__((ext_vector_type(4), aligned(2)));     // the same 16 bytes at any 2-byte element
+
+// Zero-padded copy of a rows x cols matrix of 2-byte elements (rows at any element alignment) into a
+// rows_to x cols_to one with cols_to a multiple of 8 on a 16-byte aligned base: one lane per 16-byte chunk of
+// the destination, a source chunk that lies inside its row as a whole is one 16-byte access.
+__global__ void __launch_bounds__(256) lego_pad2d_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                         unsigned rows, unsigned cols, unsigned rows_to, unsigned cols_to)
+{
+  const unsigned per_row = cols_to / 8;
+  const size_t chunk = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  const size_t r = chunk / per_row;
+  const unsigned c = static_cast<unsigned>(chunk % per_row) * 8;
+  if (r >= rows_to) return;
+  u32x4w v = {0u, 0u, 0u, 0u};
+  if (r < rows) {
+    const uint16_t* p = src + r * cols + c;
+    if (c + 8 <= cols) {
+      v = *reinterpret_cast<const u32x4w_any*>(p);
+    } else {
+#pragma unroll
+      for (unsigned e = 0; e < 8; ++e)
+        if (c + e < cols) v[e / 2] |= static_cast<uint32_t>(p[e]) << (16 * (e % 2));
+    }
+  }
+  *reinterpret_cast<u32x4w*>(dst + r * cols_to + c) = v;
+}
+
+// The way back for the result: rows x cols elements out of a matrix whose rows are cols_from elements apart.
+__global__ void __launch_bounds__(256) lego_unpad2d_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                           unsigned rows, unsigned cols, unsigned cols_from)
+{
+  const unsigned per_row = (cols + 7) / 8;
+  const size_t chunk = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  const size_t r = chunk / per_row;
+  const unsigned c = static_cast<unsigned>(chunk % per_row) * 8;
+  if (r >= rows) return;
+  const u32x4w v = *reinterpret_cast<const u32x4w*>(src + r * cols_from + c);
+  uint16_t* q = dst + r * cols + c;
+  if (c + 8 <= cols) {
+    *reinterpret_cast<u32x4w_any*>(q) = v;
+  } else {
+#pragma unroll
+    for (unsigned e = 0; e < 8; ++e)
+      if (c + e < cols) q[e] = static_cast<uint16_t>(v[e / 2] >> (16 * (e % 2)));
+  }
+}
+
+hipError_t pad2d(const void* src, void* dst, int rows, int cols, int rows_to, int cols_to, hipStream_t stream)
+{
+  const size_t chunks = static_cast<size_t>(rows_to) * (cols_to / 8);
+  hipLaunchKernelGGL(lego_pad2d_kernel, dim3(static_cast<unsigned>((chunks + 255) / 256)), dim3(256), 0, stream,
+                     static_cast<const uint16_t*>(src), static_cast<uint16_t*>(dst), static_cast<unsigned>(rows),
+                     static_cast<unsigned>(cols), static_cast<unsigned>(rows_to), static_cast<unsigned>(cols_to));
+  return hipGetLastError();
+}
+
+hipError_t unpad2d(const void* src, void* dst, int rows, int cols, int cols_from, hipStream_t stream)
+{
+  const size_t chunks = static_cast<size_t>(rows) * ((cols + 7) / 8);
+  hipLaunchKernelGGL(lego_unpad2d_kernel, dim3(static_cast<unsigned>((chunks + 255) / 256)), dim3(256), 0, stream,
+                     static_cast<const uint16_t*>(src), static_cast<uint16_t*>(dst), static_cast<unsigned>(rows),
+                     static_cast<unsigned>(cols), static_cast<unsigned>(cols_from));
+  return hipGetLastError();
+}
+
 // Scratch of lego_hip_layernorm_bwd_f16_noalloc: the fp32 dw/db partial rows that the other
 // LayerNorm backward entry points take from the caller.  One copy per device, held until the process
 // ends.  In host code the array's name is only a handle for hipGetSymbolAddress; kernels and launchers
@@ -378,9 +444,17 @@ int lego_hip_gemm_bf16_f16_ex(const void* a, const void* b, void* c, int M, int 
 int lego_hip_gemm_workspace_bytes(int M, int N, int K, unsigned long long* bytes)
 {
   if (bytes == nullptr || M <= 0 || N <= 0 || K <= 0) return kInvalid;
+  // N or K not a multiple of 8: room for zero-padded copies of both operands and of the result (2-byte elements).
+  // (M only matters as the row length of a transposed A; that case alone stays with the one-element kernel.)
+  unsigned long long copies = 0;
+  if (N % 8 || K % 8) {
+    const unsigned long long m8 = (M + 7ull) / 8 * 8, n8 = (N + 7ull) / 8 * 8, k8 = (K + 7ull) / 8 * 8;
+    copies = 2ull * (m8 * k8 + k8 * n8 + m8 * n8);
+    M = static_cast<int>(m8); N = static_cast<int>(n8); K = static_cast<int>(k8);     // the product that then runs
+  }
   const int parts = splitk_parts(M, N, K, LEGO_GEMM_BK);
   const unsigned long long tiles = static_cast<unsigned long long>((M + 127) / 128) * ((N + 127) / 128);
-  *bytes = parts > 1 ? parts * tiles * 128ull * 128ull * sizeof(float) : 0ull;
+  *bytes = copies + (parts > 1 ? parts * tiles * 128ull * 128ull * sizeof(float) : 0ull);
   return 0;
 }
 
@@ -398,7 +472,47 @@ int lego_hip_gemm_ex_ws(int element, const void* a, const void* b, void* c, int 
   // from parts, takes the plain entry point
   const bool tiled = usable(a) && usable(b) && usable(c) && N % 8 == 0 && (trans_a ? M % 8 == 0 : K % 8 == 0) &&
                      (!trans_b || K % 8 == 0);
-  if (need == 0 || !tiled || workspace == nullptr || workspace_bytes < need || !usable(workspace)) {
+  const bool have_workspace = need != 0 && workspace != nullptr && workspace_bytes >= need && usable(workspace);
+  if (have_workspace && (N % 8 || K % 8)) {
+    // Operand rows that are not whole 16-byte chunks: the tiled kernels run on zero-padded copies (every side a
+    // multiple of 8; the padding adds zeros to the sums) and the result is copied back.  Three more passes over
+    // the matrices, against the tenfold cost of the kernel that moves one element per access.
+    if (a == nullptr || b == nullptr || c == nullptr || (activation != 0 && activation != 1)) return kInvalid;
+    if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c)) & 1u) return kInvalid;
+    const int M8 = (M + 7) / 8 * 8, N8 = (N + 7) / 8 * 8, K8 = (K + 7) / 8 * 8;
+    const int Mp = trans_a ? M8 : M;                 // rows of the padded product: a transposed A has rows of M elements
+    uint16_t* ap = static_cast<uint16_t*>(workspace);
+    uint16_t* bp = ap + static_cast<size_t>(M8) * K8;
+    uint16_t* cp = bp + static_cast<size_t>(K8) * N8;
+    const bool copy_a = K8 != K || (trans_a && M8 != M) || !usable(a);
+    const bool copy_b = K8 != K || N8 != N || !usable(b);
+    const bool copy_c = N8 != N || Mp != M || !usable(c);
+    hipError_t err = hipSuccess;
+    if (copy_a) err = trans_a ? pad2d(a, ap, K, M, K8, M8, as_stream(stream)) : pad2d(a, ap, M, K, M, K8, as_stream(stream));
+    if (err != hipSuccess) return ok_or(err);
+    if (copy_b) err = trans_b ? pad2d(b, bp, N, K, N8, K8, as_stream(stream)) : pad2d(b, bp, K, N, K8, N8, as_stream(stream));
+    if (err != hipSuccess) return ok_or(err);
+    const void* aa = copy_a ? ap : a;
+    const void* bb = copy_b ? bp : b;
+    void* cc = copy_c ? cp : c;
+    int rc;
+    const int parts = splitk_parts(Mp, N8, K8, LEGO_GEMM_BK);
+    if (parts > 1) {      // few tiles: parts along K, their sums behind the copies (the size asked for covers M8 rows)
+      const splitk_launcher* by_layout = element == 0 ? f16 : element == 1 ? bf16 : bf16h;
+      rc = ok_or(by_layout[(trans_a ? 2 : 0) + (trans_b ? 1 : 0)](aa, bb, cc, Mp, N8, K8, activation, parts,
+                                                                 reinterpret_cast<float*>(cp + static_cast<size_t>(M8) * N8),
+                                                                 as_stream(stream)));
+    } else {
+      switch (element) {
+        case 0: rc = lego_hip_gemm_f16_ex(aa, bb, cc, Mp, N8, K8, trans_a, trans_b, activation, stream); break;
+        case 1: rc = lego_hip_gemm_bf16_ex(aa, bb, cc, Mp, N8, K8, trans_a, trans_b, activation, stream); break;
+        default: rc = lego_hip_gemm_bf16_f16_ex(aa, bb, cc, Mp, N8, K8, trans_a, trans_b, activation, stream); break;
+      }
+    }
+    if (rc != 0 || !copy_c) return rc;
+    return ok_or(unpad2d(cp, c, M, N, N8, as_stream(stream)));
+  }
+  if (!have_workspace || !tiled) {
     switch (element) {
       case 0: return lego_hip_gemm_f16_ex(a, b, c, M, N, K, trans_a, trans_b, activation, stream);
       case 1: return lego_hip_gemm_bf16_ex(a, b, c, M, N, K, trans_a, trans_b, activation, stream);

@@ -200,7 +200,8 @@ def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "", out_dtype=tor
         raise ValueError("out_dtype must be float16 or the operands' type")
     entry = "lego_hip_gemm_bf16_f16_ex" if (a.dtype, out_dtype) == (torch.bfloat16, torch.float16) else _GEMM_ENTRY[a.dtype]
     c = torch.empty((M, N), device=a.device, dtype=out_dtype)
-    # products of few tiles (a skinny operand, a long K) are split along K when there is room for the partial sums
+    # products of few tiles (a skinny operand, a long K) are split along K when there is room for the partial sums;
+    # shapes whose operand rows are not whole 16-byte chunks run on zero-padded copies in the workspace
     need = ctypes.c_ulonglong(0)
     runtime.call("lego_hip_gemm_workspace_bytes", M, N, K, ctypes.byref(need))
     if need.value:
