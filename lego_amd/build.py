@@ -50,7 +50,7 @@ ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f16", True, 8
            ("bf16", True, 1), ("bf16", True, 4), ("bf16", True, 8), ("bf16", True, 16), ("bf16", False, 1), ("bf16", False, 4),
            ("bf16", False, 16)]
 # (element type, lanes per row): teams of a part of a wave for rows of at most that many 16-byte vectors
-ROWWISE_SHORT = [(d, lanes) for d in ("f16", "bf16", "f32") for lanes in (16, 32)]
+ROWWISE_SHORT = [(d, lanes, vec) for d in ("f16", "bf16", "f32") for lanes in (16, 32) for vec in (True, False)]
 # LayerNorm launches of many rows: this many workgroups that stage gamma and beta in LDS and walk the rows
 ROWWISE_STREAM_WGS = {("f16", True, 8): 512, ("bf16", True, 8): 512, ("f16", True, 16): 256, ("bf16", True, 16): 256,
                       # rows of any length: a team's rows must start alike, so the count times the teams per workgroup is a multiple of 8
@@ -89,7 +89,7 @@ def collect():
             tmeta.setdefault(dtype, []).append(meta)
     units.append(transpose.emit_any())
     units += [rowwise.emit(w, dtype, vec, stream_wgs=ROWWISE_STREAM_WGS.get((dtype, vec, w), 0)) for dtype, vec, w in ROWWISE]
-    units += [rowwise.emit(1, dtype, True, team_lanes=lanes) for dtype, lanes in ROWWISE_SHORT]
+    units += [rowwise.emit(1, dtype, vec, team_lanes=lanes) for dtype, lanes, vec in ROWWISE_SHORT]
     units.append(rowwise.emit_long())
     for dtype in GEMM_DTYPES:
         for ta in (False, True):
@@ -138,9 +138,10 @@ def collect():
         h += [f"hipError_t lego_softmax_{tag}_w{w}_launch(const void*, void*, int, int, hipStream_t);",
               f"hipError_t lego_layernorm_fwd_{tag}_w{w}_launch(const void*, void*, const void*, const void*, "
               "float*, float*, int, int, float, hipStream_t);"]
-    for dtype, lanes in ROWWISE_SHORT:
-        h += [f"hipError_t lego_softmax_{dtype}_l{lanes}_launch(const void*, void*, int, int, hipStream_t);",
-              f"hipError_t lego_layernorm_fwd_{dtype}_l{lanes}_launch(const void*, void*, const void*, const void*, "
+    for dtype, lanes, vec in ROWWISE_SHORT:
+        tag = dtype if vec else dtype + "s"
+        h += [f"hipError_t lego_softmax_{tag}_l{lanes}_launch(const void*, void*, int, int, hipStream_t);",
+              f"hipError_t lego_layernorm_fwd_{tag}_l{lanes}_launch(const void*, void*, const void*, const void*, "
               "float*, float*, int, int, float, hipStream_t);"]
     h += [f"hipError_t lego_softmax_long_{d}_launch(const void*, void*, int, int, hipStream_t);" for d in rowwise.ELEMENTS]
     h += [

@@ -178,7 +178,8 @@ int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream)
   if (N > LEGO_ROWWISE_MAX_N) return ok_or(lego_softmax_long_f16_launch(x, y, M, N, as_stream(stream)));   // two passes
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 8)   // ragged rows
-    return ok_or((long_row ? lego_softmax_f16s_w16_launch : lego_rowwise_default_wpr(N) == 1 ? lego_softmax_f16s_w1_launch
+    return ok_or((N <= 128 ? lego_softmax_f16s_l16_launch : N <= 256 ? lego_softmax_f16s_l32_launch
+                  : long_row ? lego_softmax_f16s_w16_launch : lego_rowwise_default_wpr(N) == 1 ? lego_softmax_f16s_w1_launch
                                                                                            : lego_softmax_f16s_w4_launch)(
         x, y, M, N, as_stream(stream)));
   return lego_hip_softmax_f16_wpr(x, y, M, N, lego_rowwise_f16_wpr(M, N), stream);
@@ -190,7 +191,8 @@ int lego_hip_softmax_f32(const void* x, void* y, int M, int N, void* stream)
   if (N > LEGO_ROWWISE_MAX_N) return ok_or(lego_softmax_long_f32_launch(x, y, M, N, as_stream(stream)));   // two passes
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 4)   // ragged rows
-    return ok_or((long_row ? lego_softmax_f32s_w16_launch : N <= 1024 ? lego_softmax_f32s_w1_launch
+    return ok_or((N <= 64 ? lego_softmax_f32s_l16_launch : N <= 128 ? lego_softmax_f32s_l32_launch
+                  : long_row ? lego_softmax_f32s_w16_launch : N <= 1024 ? lego_softmax_f32s_w1_launch
                                                                       : lego_softmax_f32s_w4_launch)(x, y, M, N, as_stream(stream)));
   if (N <= 1024)   // rows of at most 16 or 32 vectors: several rows per wave
     return ok_or((N <= 64 ? lego_softmax_f32_l16_launch : N <= 128 ? lego_softmax_f32_l32_launch : lego_softmax_f32_w1_launch)(
@@ -224,7 +226,8 @@ int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void
   if (M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 8)   // ragged rows
-    return ok_or((long_row ? lego_layernorm_fwd_f16s_w16_launch : lego_rowwise_default_wpr(N) == 1 ? lego_layernorm_fwd_f16s_w1_launch
+    return ok_or((N <= 128 ? lego_layernorm_fwd_f16s_l16_launch : N <= 256 ? lego_layernorm_fwd_f16s_l32_launch
+                  : long_row ? lego_layernorm_fwd_f16s_w16_launch : lego_rowwise_default_wpr(N) == 1 ? lego_layernorm_fwd_f16s_w1_launch
                                                                                                  : lego_layernorm_fwd_f16s_w4_launch)(
         x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
   return lego_hip_layernorm_fwd_f16_wpr(x, y, w, b, mean, rstd, M, N, eps, lego_rowwise_f16_wpr(M, N), stream);
@@ -237,7 +240,8 @@ int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void
   if (M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 4)   // ragged rows
-    return ok_or((long_row ? lego_layernorm_fwd_f32s_w16_launch : N <= 1024 ? lego_layernorm_fwd_f32s_w1_launch
+    return ok_or((N <= 64 ? lego_layernorm_fwd_f32s_l16_launch : N <= 128 ? lego_layernorm_fwd_f32s_l32_launch
+                  : long_row ? lego_layernorm_fwd_f32s_w16_launch : N <= 1024 ? lego_layernorm_fwd_f32s_w1_launch
                                                                             : lego_layernorm_fwd_f32s_w4_launch)(
         x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
   if (N <= 1024)
@@ -254,7 +258,8 @@ int lego_hip_softmax_bf16(const void* x, void* y, int M, int N, void* stream)
   if (N > LEGO_ROWWISE_MAX_N) return ok_or(lego_softmax_long_bf16_launch(x, y, M, N, as_stream(stream)));   // two passes
   const int wpr = lego_rowwise_default_wpr(N);
   if (N % 8)   // ragged rows
-    return ok_or((wpr == 16 ? lego_softmax_bf16s_w16_launch : wpr == 1 ? lego_softmax_bf16s_w1_launch
+    return ok_or((N <= 128 ? lego_softmax_bf16s_l16_launch : N <= 256 ? lego_softmax_bf16s_l32_launch
+                  : wpr == 16 ? lego_softmax_bf16s_w16_launch : wpr == 1 ? lego_softmax_bf16s_w1_launch
                                                                        : lego_softmax_bf16s_w4_launch)(x, y, M, N, as_stream(stream)));
   if (N <= 256) return ok_or((N <= 128 ? lego_softmax_bf16_l16_launch : lego_softmax_bf16_l32_launch)(x, y, M, N, as_stream(stream)));
   if (lego_rowwise_f16_wpr(M, N) == 8) return ok_or(lego_softmax_bf16_w8_launch(x, y, M, N, as_stream(stream)));   // as fp16
@@ -269,7 +274,8 @@ int lego_hip_layernorm_fwd_bf16(const void* x, void* y, const void* w, const voi
   if (M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
   const int wpr = lego_rowwise_default_wpr(N);
   if (N % 8)   // ragged rows
-    return ok_or((wpr == 16 ? lego_layernorm_fwd_bf16s_w16_launch : wpr == 1 ? lego_layernorm_fwd_bf16s_w1_launch
+    return ok_or((N <= 128 ? lego_layernorm_fwd_bf16s_l16_launch : N <= 256 ? lego_layernorm_fwd_bf16s_l32_launch
+                  : wpr == 16 ? lego_layernorm_fwd_bf16s_w16_launch : wpr == 1 ? lego_layernorm_fwd_bf16s_w1_launch
                                                                              : lego_layernorm_fwd_bf16s_w4_launch)(
         x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
   if (N <= 256)

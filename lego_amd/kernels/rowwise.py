@@ -41,7 +41,7 @@ def emit(waves_per_row=1, dtype="f16", vectorised=True, seq_max_wpr=4, prefetch_
     TEAM = 64 * WPR
     wtag = f"w{WPR}"
     if team_lanes:
-        assert WPR == 1 and vectorised and team_lanes in (16, 32)
+        assert WPR == 1 and team_lanes in (16, 32)
         TEAM, wtag = team_lanes, f"l{team_lanes}"
     threads = max(THREADS, TEAM)
     RPW = threads // TEAM                       # rows per workgroup

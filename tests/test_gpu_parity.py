@@ -394,7 +394,9 @@ def test_layernorm_backward_fp32(ops, M, N):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("M,N", [(1, 8), (37, 24), (300, 64), (77, 120), (1000, 128), (41, 136), (513, 248), (260, 256)])
+@pytest.mark.parametrize("M,N", [(1, 8), (37, 24), (300, 64), (77, 120), (1000, 128), (41, 136), (513, 248), (260, 256),
+                                 # of any length: head and tail elements on the first lanes of the team
+                                 (64, 7), (37, 25), (300, 63), (77, 121), (1000, 127), (41, 129), (513, 250), (260, 255)])
 def test_short_rows_share_a_wave(ops, dtype, M, N):
     """Rows of at most 16 or 32 vectors are dealt 4 or 2 to a wave (teams of 16 or 32 lanes, 16 or 8 rows per
     workgroup, LayerNorm two rows per team): row counts that leave teams and workgroups partly empty, row
