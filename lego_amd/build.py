@@ -108,8 +108,8 @@ def collect():
                                       with_grouped=dtype == "f16" and not (ta or tb), with_splitk=True)
                     units.append(gs)
     units.append(gemm.emit_any())
-    lb, mlb = layernorm_bwd.emit()
-    units.append(lb)
+    lbs, mlb = layernorm_bwd.emit()
+    units += lbs
     nwu, mnw = nw.emit()
     units.append(nwu)
     stu, mst = stencil.emit()

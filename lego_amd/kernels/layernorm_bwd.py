@@ -35,7 +35,15 @@ WAVE_MAX_N = 1024
 WAVE_GROUPS = 1024    # workgroups of those kernels = rows of their partial buffers
 
 
+ELTS = (("_Float16", "f16", "half8"), ("__bf16", "bf16", "bhalf8"), ("float", "f32", "float8v"))
+
+
 def emit():
+    """One translation unit per element type (they compile side by side); ``(units, constants)``."""
+    return [_emit(elt) for elt in ELTS], dict(MAX_N=LONG[0] * LONG[1] * 8, MAX_GROUPS=MAX_GROUPS)
+
+
+def _emit(elt):
     M, N, G, STEPS = size("M"), size("N"), size("G"), size("STEPS")
     wg, t, it, step, row, v = (idx(n) for n in ("wg", "t", "it", "step", "row", "v"))
     rows = OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])
@@ -50,7 +58,7 @@ def emit():
         RAGGED_CONFIGS=list(RAGGED_CONFIGS), RAGGED_MAX_N_256=max(v for th, v in RAGGED_CONFIGS if th == 256) * 256 * 8,
         WAVE_VS=WAVE_VS, WAVE_MAX_N=WAVE_MAX_N, WAVE_GROUPS=WAVE_GROUPS,
         # every element type takes the same kernels, eight elements per lane and step: (type, tag, vector type)
-        ELTS=[("_Float16", "f16", "half8"), ("__bf16", "bf16", "bhalf8"), ("float", "f32", "float8v")],
+        ELTS=[elt], WITH_GROUPS=elt[1] == "f16",
         MAX_N_ACC=max(th * v for th, v in CONFIGS) * 8,
         MAX_N_256=max(v for th, v in CONFIGS if th == 256) * 256 * 8,
         row_layout="OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])[step, wg]",
@@ -65,5 +73,4 @@ def emit():
         part_off=code(tidy(P[wg, v, 0, 0], {wg: (0, G), v: (0, N / 8)})).replace("wg", "static_cast<size_t>(wg)"),
     )
     text = template("layernorm_bwd.hip.j2").render(**params)
-    return Emitted("layernorm_bwd_f16.hip", text, ["lego_layernorm_bwd_f16_launch", "lego_layernorm_bwd_f32_launch", "lego_layernorm_bwd_bf16_launch"]), dict(
-        MAX_N=LONG[0] * LONG[1] * 8, MAX_GROUPS=MAX_GROUPS)
+    return Emitted(f"layernorm_bwd_{elt[1]}.hip", text, [f"lego_layernorm_bwd_{elt[1]}_launch"])
