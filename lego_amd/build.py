@@ -33,7 +33,7 @@ TRANSPOSE = {
             dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag"),
             dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag"),
             dict(dtype="f32", tile=(32, 32), group=(2, 4), order="diag", edge=True),
-            dict(dtype="f32", tile=(32, 32), group=(2, 4), order="diag", edge=True, ragged=True)],
+            dict(dtype="f32", tile=(32, 32), group=(4, 2), order="diag", edge=True, ragged=True)],
     "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 128, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 64, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 32, 8)),
