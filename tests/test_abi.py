@@ -53,3 +53,35 @@ def test_argument_validation_needs_no_gpu():
 def test_missing_library_fails_loudly(tmp_path):
     with pytest.raises(FileNotFoundError):
         runtime.load_library(tmp_path / "liblego_hip.so")
+
+
+def test_workspace_sizes_follow_the_launch_rules():
+    """The size queries are plain host functions.  LayerNorm backward: the partial rows are `N` rounded up to 8
+    floats apart; when rows of any length are walked by fewer workgroups than rows, the number of workgroups is
+    a multiple of eight, so that a workgroup's rows start at the same offset from a 16-byte boundary.  GEMM: a
+    shape with N or K off the 16-byte grid asks for room for padded copies of both operands and the result."""
+    lib = runtime.load_library()
+    need = ctypes.c_ulonglong(0)
+    for entry, elements_per_16_bytes in (("lego_hip_layernorm_bwd_workspace_bytes", 8),
+                                         ("lego_hip_layernorm_bwd_bf16_workspace_bytes", 8),
+                                         ("lego_hip_layernorm_bwd_f32_workspace_bytes", 4)):
+        fn = getattr(lib, entry)
+        for N in (1, 7, 33, 250, 781, 1001, 1023, 2050, 4099, 8191, 12001, 16383, 512, 4096, 16384):
+            pitch = (N + 7) // 8 * 8
+            for M in (1, 3, 8, 100, 255, 256, 257, 511, 513, 1000, 4097, 100000):
+                assert fn(M, N, ctypes.byref(need)) == 0
+                assert need.value % (2 * pitch * 4) == 0
+                groups = need.value // (2 * pitch * 4)
+                assert 1 <= groups <= max(M, 8) and groups <= 1024, (entry, M, N, groups)
+                if N % 8 and groups < M:
+                    assert groups % 8 == 0, (entry, M, N, groups)
+                if N % 8 and N <= 1024:       # a wavefront per row: the four waves of a workgroup start alike too
+                    assert groups % 8 == 0, (entry, M, N, groups)
+        assert fn(4, 32769, ctypes.byref(need)) == 1 and fn(0, 8, ctypes.byref(need)) == 1
+    for M, N, K in ((193, 131, 77), (4096, 4096, 4097), (4096, 4100, 4096), (5, 7, 3), (16, 8190, 8192)):
+        assert lib.lego_hip_gemm_workspace_bytes(M, N, K, ctypes.byref(need)) == 0
+        r8 = lambda v: (v + 7) // 8 * 8
+        assert need.value >= 2 * (r8(M) * r8(K) + r8(K) * r8(N) + r8(M) * r8(N)), (M, N, K)
+        assert need.value % 16 == 0
+    for M, N, K in ((4096, 4096, 4096), (1001, 264, 200), (2048, 1024, 64)):     # M alone never asks for copies
+        assert lib.lego_hip_gemm_workspace_bytes(M, N, K, ctypes.byref(need)) == 0 and need.value == 0, (M, N, K)
