@@ -403,11 +403,13 @@ int gemm_ex(const GemmKernels& k, int element, const void* a, const void* b, voi
 }
 
 // Parts along K for a product of few tiles (1: one workgroup per tile does it all): enough parts for two
-// workgroups of 128 x 128 tiles per CU, at least four k-tiles each.
+// workgroups of 128 x 128 tiles per CU, at least four k-tiles each.  The second launch and the partial sums cost
+// about what 16 k-tiles take, so shallower products stay whole (1024^3: 8.6 us whole, 11.7 in four parts;
+// 512 x 512 x 2048: 13.7 whole, 8.2 in eight).
 int splitk_parts(int M, int N, int K, int bk)
 {
   const long tiles = static_cast<long>((M + 127) / 128) * ((N + 127) / 128), depth = (K + bk - 1) / bk;
-  if (tiles > 128 || depth < 8) return 1;
+  if (tiles > 128 || depth < 32) return 1;
   long parts = (512 + tiles - 1) / tiles;
   if (parts > depth / 4) parts = depth / 4;
   if (parts > 64) parts = 64;
