@@ -199,6 +199,10 @@ def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "", out_dtype=tor
     if out_dtype not in (torch.float16, a.dtype):
         raise ValueError("out_dtype must be float16 or the operands' type")
     entry = "lego_hip_gemm_bf16_f16_ex" if (a.dtype, out_dtype) == (torch.bfloat16, torch.float16) else _GEMM_ENTRY[a.dtype]
+    if ta and M % 8 and M * K >= 65536:
+        # a column-major A whose columns (M elements) are not whole 16-byte chunks is outside the tiled kernels whatever
+        # the workspace: store it row-major first (one pass with the transpose kernels)
+        a_store, ta = transpose(a_store), 0
     c = torch.empty((M, N), device=a.device, dtype=out_dtype)
     # products of few tiles (a skinny operand, a long K) are split along K when there is room for the partial sums;
     # shapes whose operand rows are not whole 16-byte chunks run on zero-padded copies in the workspace
