@@ -63,6 +63,7 @@ ROWWISE_MAX_N = rowwise.MAX_N
 GEMM = dict(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8)
 GEMM_SMALL_TILE = 128
 GEMM_SMALL_DTYPES = ("f16", "bf16", "bf16h")     # a 128-byte row of 8-bit elements is too short for their [k][n] rotation
+GEMM_SMALL_NT_ONLY = ("e4m3", "e5m2")             # ... so 8-bit operands get the small tile where both are k-major (A as given, B transposed)
 GEMM_DTYPES = ("f16", "bf16", "bf16h", "e4m3", "e5m2")     # bf16h: bfloat16 operands, fp16 result
 GEMM_BK = {"f16": 64, "bf16": 64, "bf16h": 64, "e4m3": 128, "e5m2": 128}   # 128 bytes of k per operand row in every case
 
@@ -106,6 +107,10 @@ def collect():
                     gs, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK[dtype], bm=GEMM_SMALL_TILE, bn=GEMM_SMALL_TILE),
                                       trans_a=ta, trans_b=tb, dtype=dtype,
                                       with_grouped=dtype == "f16" and not (ta or tb), with_splitk=True)
+                    units.append(gs)
+                elif dtype in GEMM_SMALL_NT_ONLY and tb and not ta:
+                    gs, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK[dtype], bm=GEMM_SMALL_TILE, bn=GEMM_SMALL_TILE),
+                                      trans_a=ta, trans_b=tb, dtype=dtype, with_grouped=False)
                     units.append(gs)
     units.append(gemm.emit_any())
     lbs, mlb = layernorm_bwd.emit()
@@ -167,7 +172,7 @@ def collect():
           f"#define LEGO_LAYERNORM_BWD_MAX_N {mlb['MAX_N']}", ""]
     h += [f"hipError_t lego_gemm_{d}_{v}{t}_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);"
           for d in GEMM_DTYPES for v in ("nn", "nt", "tn", "tt")
-          for t in ("", f"_t{GEMM_SMALL_TILE}x{GEMM_SMALL_TILE}") if not t or d in GEMM_SMALL_DTYPES]
+          for t in ("", f"_t{GEMM_SMALL_TILE}x{GEMM_SMALL_TILE}") if not t or d in GEMM_SMALL_DTYPES or (d in GEMM_SMALL_NT_ONLY and v == "nt")]
     h += [f"hipError_t lego_gemm_{d}_{v}_t{GEMM_SMALL_TILE}x{GEMM_SMALL_TILE}_splitk_launch(const void*, const void*, void*, int, int, int, int, "
           "int, float*, hipStream_t);" for d in GEMM_SMALL_DTYPES for v in ("nn", "nt", "tn", "tt")]
     h += [

@@ -398,8 +398,9 @@ int gemm_ex(const GemmKernels& k, int element, const void* a, const void* b, voi
                                       as_stream(stream)));
   }
   const long tiles = static_cast<long>((M + LEGO_GEMM_BM - 1) / LEGO_GEMM_BM) * ((N + LEGO_GEMM_BN - 1) / LEGO_GEMM_BN);
-  const gemm_launcher* by_layout = tiles < kSmallTileBelow && k.small[0] != nullptr ? k.small : k.big;
-  return ok_or(by_layout[(trans_a ? 2 : 0) + (trans_b ? 1 : 0)](a, b, c, M, N, K, activation, as_stream(stream)));
+  const int layout = (trans_a ? 2 : 0) + (trans_b ? 1 : 0);
+  const gemm_launcher* by_layout = tiles < kSmallTileBelow && k.small[layout] != nullptr ? k.small : k.big;
+  return ok_or(by_layout[layout](a, b, c, M, N, K, activation, as_stream(stream)));
 }
 
 // Parts along K for a product of few tiles (1: one workgroup per tile does it all): enough parts for two
@@ -417,10 +418,11 @@ int splitk_parts(int M, int N, int K, int bk)
 }
 typedef hipError_t (*splitk_launcher)(const void*, const void*, void*, int, int, int, int, int, float*, hipStream_t);
 
-#define LEGO_GEMM_KERNELS_BIG_ONLY(DT)                                                                 \
+// 8-bit operands: the small tile only where both operands are k-major (A as given, B transposed)
+#define LEGO_GEMM_KERNELS_SMALL_NT(DT)                                                                 \
   {{lego_gemm_##DT##_nn_launch, lego_gemm_##DT##_nt_launch, lego_gemm_##DT##_tn_launch,              \
     lego_gemm_##DT##_tt_launch},                                                                       \
-   {nullptr, nullptr, nullptr, nullptr}}
+   {nullptr, lego_gemm_##DT##_nt_t128x128_launch, nullptr, nullptr}}
 #define LEGO_GEMM_KERNELS(DT)                                                                          \
   {{lego_gemm_##DT##_nn_launch, lego_gemm_##DT##_nt_launch, lego_gemm_##DT##_tn_launch,              \
     lego_gemm_##DT##_tt_launch},                                                                       \
@@ -536,8 +538,8 @@ int lego_hip_gemm_ex_ws(int element, const void* a, const void* b, void* c, int 
 int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                          int activation, int format, void* stream)
 {
-  static const GemmKernels e4m3 = LEGO_GEMM_KERNELS_BIG_ONLY(e4m3);
-  static const GemmKernels e5m2 = LEGO_GEMM_KERNELS_BIG_ONLY(e5m2);
+  static const GemmKernels e4m3 = LEGO_GEMM_KERNELS_SMALL_NT(e4m3);
+  static const GemmKernels e5m2 = LEGO_GEMM_KERNELS_SMALL_NT(e5m2);
   if (format != 0 && format != 1) return kInvalid;
   return gemm_ex(format == 0 ? e4m3 : e5m2, format == 0 ? 2 : 3, a, b, c, M, N, K, trans_a, trans_b, activation,
                  stream, LEGO_GEMM_BK_8BIT, 16);
