@@ -28,8 +28,8 @@ OBJ_DIR = LIB_DIR / "obj"
 # divide (then the same in smaller windows), a wide macro tile in skewed ("diag") order, a 64x64 one for shapes the wide tile
 # does not divide, and the wide tile with edge tests for shapes in whole 16-byte vectors.
 TRANSPOSE = {
-    "f32": [dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 64, 8), max_bytes=256 << 20),
-            dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 32, 8), max_bytes=256 << 20),
+    "f32": [dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 64, 8), max_bytes=1536 << 20),
+            dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 32, 8), max_bytes=1536 << 20),
             dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag"),
             dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag"),
             dict(dtype="f32", tile=(32, 32), group=(2, 4), order="diag", edge=True),
