@@ -197,6 +197,9 @@ int lego_hip_softmax_f32(const void* x, void* y, int M, int N, void* stream)
   if (N <= 1024)   // rows of at most 16 or 32 vectors: several rows per wave
     return ok_or((N <= 64 ? lego_softmax_f32_l16_launch : N <= 128 ? lego_softmax_f32_l32_launch : lego_softmax_f32_w1_launch)(
         x, y, M, N, as_stream(stream)));
+  // eight waves for the rows that take them in the 16-bit types, by their bytes (8192^2: softmax +3 %, LayerNorm +6 %;
+  // 16384 x 4096 +6 % and +2 %)
+  if (lego_rowwise_f16_wpr(M, 2 * N) == 8) return ok_or(lego_softmax_f32_w8_launch(x, y, M, N, as_stream(stream)));
   return ok_or((long_row ? lego_softmax_f32_w16_launch : lego_softmax_f32_w4_launch)(x, y, M, N, as_stream(stream)));
 }
 
@@ -248,6 +251,8 @@ int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void
     return ok_or((N <= 64 ? lego_layernorm_fwd_f32_l16_launch : N <= 128 ? lego_layernorm_fwd_f32_l32_launch
                                                                       : lego_layernorm_fwd_f32_w1_launch)(
         x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
+  if (lego_rowwise_f16_wpr(M, 2 * N) == 8)   // as the 16-bit types, by the bytes of a row
+    return ok_or(lego_layernorm_fwd_f32_w8_launch(x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
   return ok_or((long_row ? lego_layernorm_fwd_f32_w16_launch : lego_layernorm_fwd_f32_w4_launch)(
       x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
 }

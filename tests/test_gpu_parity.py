@@ -205,7 +205,9 @@ def test_softmax_reference_test_shape_fp32(ops):
                                  (3, 16392), (2, 20001), (5, 32767), (4, 32768),
                                  # tall and ragged: teams walk rows that start alike, the next row's loads in flight
                                  (8300, 781), (8195, 250), (8200, 1001), (2050, 4099), (2049, 8191), (2300, 2050),
-                                 (1030, 12001), (1100, 16383), (515, 20001), (600, 32767)])
+                                 (1030, 12001), (1100, 16383), (515, 20001), (600, 32767),
+                                 # tall, rows of 12-32 KiB: teams of eight waves in fp32 as well
+                                 (4100, 4096), (4097, 8192), (4096, 3076)])
 def test_softmax_ragged_and_fp32(ops, dtype, M, N):
     print(f"softmax {dtype} {M}x{N}", flush=True)
     x = (2.0 * torch.randn(M, N, generator=_gen(2))).to(dtype)
@@ -219,7 +221,9 @@ def test_softmax_ragged_and_fp32(ops, dtype, M, N):
                                  (4, 32768),
                                  # tall and ragged: teams walk rows that start alike, gamma and beta shifted into LDS
                                  (8300, 781), (8195, 250), (8200, 1001), (2050, 4099), (2049, 8191), (2300, 2050),
-                                 (515, 20001), (600, 32767), (1030, 12001), (1100, 16383), (4100, 3001)])
+                                 (515, 20001), (600, 32767), (1030, 12001), (1100, 16383), (4100, 3001),
+                                 # tall, rows of 12-32 KiB: teams of eight waves in fp32 as well (gamma and beta in LDS)
+                                 (4100, 4096), (4097, 8192), (4096, 3076)])
 def test_layernorm_ragged_and_fp32(ops, dtype, M, N):
     print(f"layernorm {dtype} {M}x{N}", flush=True)
     if N * torch.empty((), dtype=dtype).element_size() > 65536:
