@@ -77,6 +77,7 @@ def emit(waves_per_row=1, dtype="f16", vectorised=True, seq_max_wpr=4, prefetch_
         dtype=dtype, elt=elt, EPV=EPV, ESIZE=esize, RAGGED=not vectorised, tag=tag,
         SEQ_MAX_WPR=seq_max_wpr, PREFETCH_MAX_WPR=prefetch_max_wpr,
         STREAM=stream_wgs > 0 and (RPW == 1 or not vectorised), STREAM_WGS=stream_wgs,
+        WALK_STEPS=64 if vectorised else 16,     # rows per team and launch of the walking kernels
         stream_team_layout=f"OrderBy(Row(STEPS, G, {RPW})).TileBy([STEPS], [G], [{RPW}])[step, wg, team]",
         stream_team_row=code(stream_team_row), stream_team0_row=code(stream_team0_row),
         stream_layout="OrderBy(Row(STEPS, G)).TileBy([STEPS], [G])[step, wg]", stream_row=code(stream_row),

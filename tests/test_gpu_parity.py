@@ -246,6 +246,31 @@ def test_layernorm_ragged_and_fp32(ops, dtype, M, N):
         assert torch.allclose(rstd.cpu(), want_rstd, atol=1e-4, rtol=1e-3)
 
 
+@pytest.mark.parametrize("M,N", [(24600, 8191), (201500, 1001)])
+def test_rows_of_any_length_results_past_the_cache(ops, M, N):
+    """fp16 results of more than 384 MiB: the kernels for rows of any length store them with non-temporal
+    stores (another instantiation), the walking kernels in launches of at most 16 rows per team.  At this size:
+    row sums of the softmax, the statistics against torch on the GPU, and the first and last rows (the ends of
+    the first and of the last launch) against the oracle."""
+    print(f"rows of any length, large result {M}x{N}", flush=True)
+    assert M * N * 2 > 384 << 20
+    g = _gen(61)
+    xd = (2.0 * torch.randn(M, N, generator=g, dtype=torch.float32)).half().cuda()
+    w = (1 + 0.1 * torch.randn(N, generator=g)).half()
+    b = (0.1 * torch.randn(N, generator=g)).half()
+    sm = ops.softmax(xd)
+    assert (sm.float().sum(-1) - 1).abs().max().item() <= 2e-2
+    y, mean, rstd = ops.layer_norm_fwd(xd, w.cuda(), b.cuda(), 1e-5)
+    xf = xd.float()
+    assert (mean - xf.mean(-1)).abs().max().item() <= 1e-4
+    assert ((rstd - torch.rsqrt(xf.var(-1, unbiased=False) + 1e-5)).abs() <= 1e-3 * rstd.abs()).all()
+    del xf
+    for rows in (slice(0, 48), slice(M // 2 - 24, M // 2 + 24), slice(M - 48, M)):
+        x = xd[rows].cpu()
+        assert (sm[rows].cpu().float() - ok.softmax(x).float()).abs().max().item() <= TOL
+        _assert_layernorm_forward(y[rows], x, w, b)
+
+
 @pytest.mark.parametrize("N", [16392, 30001, 32768])
 def test_layernorm_fp32_long_rows_through_the_c_abi(ops, N):
     """fp32 rows above 64 KiB: the Python wrapper keeps the reference's limit, the library takes them."""
