@@ -32,15 +32,15 @@ TRANSPOSE = {
             dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 32, 8), max_bytes=1536 << 20),
             dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag"),
             dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag"),
-            dict(dtype="f32", tile=(32, 32), group=(2, 4), order="diag", edge=True),
-            dict(dtype="f32", tile=(32, 32), group=(4, 2), order="diag", edge=True, ragged=True)],
+            dict(dtype="f32", tile=(32, 32), group=(2, 4), order="col", edge=True, xcd=True),
+            dict(dtype="f32", tile=(32, 32), group=(4, 2), order="col", edge=True, ragged=True, xcd=True)],
     "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 128, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 64, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 32, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag"),
             dict(dtype="f16", tile=(64, 64), group=(1, 1), order="diag"),
-            dict(dtype="f16", tile=(64, 64), group=(2, 2), order="diag", edge=True),
-            dict(dtype="f16", tile=(64, 64), group=(2, 2), order="diag", edge=True, ragged=True)],
+            dict(dtype="f16", tile=(64, 64), group=(2, 2), order="col", edge=True, xcd=True),
+            dict(dtype="f16", tile=(64, 64), group=(2, 2), order="col", edge=True, ragged=True, xcd=True)],
 }
 # (element type, vectorised, waves per row): 16-byte accesses need N % (16/size) == 0; the
 # element-per-access kernels ("s") take any N

@@ -132,11 +132,12 @@ def tile_order(order, n_bi, n_bj, wg):
     raise ValueError(order)
 
 
-def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix="", edge=False, ragged=False):
+def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix="", edge=False, ragged=False, xcd=False):
     """HIP translation unit for one element type and one tiling.  ``edge``: the shape need not be
     a whole number of macro tiles, only of 16-byte vectors in both directions; vectors past the
     edge are skipped.  ``ragged`` (with ``edge``): any shape; rows start at any element, the vectors
-    that an edge cuts go element by element."""
+    that an edge cuts go element by element.  ``xcd`` (with ``edge``): workgroup ids are dealt to the tiles
+    so that each XCD takes a contiguous run of them (``order`` is then the order inside that run)."""
     elt, esize = {"f32": ("float", 4), "f16": ("_Float16", 2)}[dtype]
     vec = 16 // esize                       # elements per 16-byte vector
     (TR, TC), (MR, MC) = tile, group
@@ -183,7 +184,7 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix="", edge=
     if edge:
         assert not windowed
         suffix = f"{suffix}_ragged" if ragged else f"{suffix}_edge"
-    assert edge or not ragged
+    assert edge or not (ragged or xcd)
     rng1 = {r: (0, SR), cv: (0, SC // vec), e: (0, 4)}
     rng2 = {k: (0, KD), rv: (0, SR // rows_per_read)}
     cols_per_word = 4 // esize
@@ -202,7 +203,9 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix="", edge=
         lds_load1=code(tidy(lds[k, rv * rows_per_read + 4], rng2)) if esize == 2 else "",
         dst_off0=code(in_tile(dst, rv * rows_per_read, k * cols_per_word, rng2)),
         dst_off1=code(in_tile(dst, rv * rows_per_read, k * cols_per_word + 1, rng2)) if esize == 2 else "",
-        grid=(f"static_cast<unsigned>((rows + {SR - 1}) / {SR}) * static_cast<unsigned>((cols + {SC - 1}) / {SC})" if edge
+        xcd=xcd,
+        grid=(f"(static_cast<unsigned>((rows + {SR - 1}) / {SR}) * static_cast<unsigned>((cols + {SC - 1}) / {SC}) + 7) / 8 * 8" if edge and xcd else
+              f"static_cast<unsigned>((rows + {SR - 1}) / {SR}) * static_cast<unsigned>((cols + {SC - 1}) / {SC})" if edge
               else f"static_cast<unsigned>(rows / {SR}) * static_cast<unsigned>(cols / {SC})"),
         edge=edge, ragged=ragged, VEC=vec, bits_t="uint32_t" if esize == 4 else "uint16_t",
         # matrix coordinates of the vectors, for the edge tests: source (row, first column) in phase 1,
