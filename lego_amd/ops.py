@@ -222,13 +222,27 @@ def lego_group_gemm_fn(group_A, group_B):
     """One launch for a list of independent GEMMs; returns the list of results."""
     if len(group_A) != len(group_B):
         raise ValueError("group_A and group_B must have the same length")
-    groups = len(group_A)
-    group_C, sizes = [], []
     for a, b in zip(group_A, group_B):
         _check(a, torch.float16, "A")
         _check(b, torch.float16, "B")
         if a.shape[1] != b.shape[0]:
             raise ValueError("Incompatible dimensions")
+    # Problems whose rows are not whole 16-byte chunks would take the whole call to one launch per problem with the
+    # one-element kernel: those few go through ``matmul`` (zero-padded copies, a workspace from torch), the rest in
+    # one launch.
+    odd = [i for i, b in enumerate(group_B) if b.shape[0] % 8 or b.shape[1] % 8]
+    if odd:
+        rest = [i for i in range(len(group_A)) if i not in set(odd)]
+        out = [None] * len(group_A)
+        if rest:
+            for i, c in zip(rest, lego_group_gemm_fn([group_A[i] for i in rest], [group_B[i] for i in rest])):
+                out[i] = c
+        for i in odd:
+            out[i] = matmul(group_A[i], group_B[i])
+        return out
+    groups = len(group_A)
+    group_C, sizes = [], []
+    for a, b in zip(group_A, group_B):
         M, K = a.shape
         N = b.shape[1]
         group_C.append(torch.empty((M, N), device=a.device, dtype=a.dtype))
