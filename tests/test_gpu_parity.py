@@ -717,6 +717,26 @@ def test_grouped_gemm_with_odd_problems(ops):
         assert ((c.cpu().float() - w.float()).abs() <= 2.0 ** -9 * w.float().abs() + 1e-3).all()
 
 
+def test_grouped_gemm_entry_point_with_odd_problems(ops):
+    """The C entry point itself (the wrapper sends odd problems elsewhere): a call with problems outside the tiled
+    kernels falls back to one launch per problem, small integers bit for bit."""
+    import ctypes
+    from lego_amd import runtime
+    print("grouped gemm entry point, odd problems", flush=True)
+    g = _gen(46)
+    shapes = [(256, 128, 64), (101, 63, 50), (64, 72, 200), (7, 5, 3)]
+    A = [torch.randint(-2, 3, (m, k), generator=g).half().cuda() for m, n, k in shapes]
+    B = [torch.randint(-2, 3, (k, n), generator=g).half().cuda() for m, n, k in shapes]
+    C = [torch.empty(m, n, dtype=torch.half, device="cuda") for m, n, k in shapes]
+    arr = ctypes.c_void_p * len(shapes)
+    sz = (ctypes.c_int * (3 * len(shapes)))(*[v for s3 in shapes for v in s3])
+    runtime.call("lego_hip_grouped_gemm_f16", arr(*[t.data_ptr() for t in A]), arr(*[t.data_ptr() for t in B]),
+                 arr(*[t.data_ptr() for t in C]), sz, len(shapes), None)
+    torch.cuda.synchronize()
+    for a, b, c in zip(A, B, C):
+        assert torch.equal(c.float(), a.float() @ b.float())
+
+
 def test_grouped_gemm_takes_up_to_64_problems(ops):
     """The most problems one call takes (the kernels' argument block holds 64), all of different shape, many of a
     single ragged tile; one more is refused."""
