@@ -159,8 +159,11 @@ def collect():
           f"{ROWWISE_DEFAULT_WAVES} : {rowwise.LONG_ROW_WAVES}; }}",
           "// 16-bit rows of whole vectors: eight waves (a workgroup of 512 lanes, two to four vectors per lane) for long",
           "// rows of tall matrices, where they measure 3-5 % above four waves; fewer rows leave too few workgroups",
+          "// ... and two waves (two rows per workgroup) for 2049-4096 rows of 2049-4096 elements: one round of workgroups on",
+          "// the 256 CUs instead of two (4096 x 4096: softmax 4.9 -> 5.4 TB/s, LayerNorm 4.4 -> 5.0; no gain from 8192 rows on)",
           f"inline int lego_rowwise_f16_wpr(int m, int n) {{ return n > {ROWWISE_WIDE_TEAM_ABOVE_N} && n <= "
-          f"{rowwise.MAX_N_SMALL_TEAMS} && m >= {ROWWISE_WIDE_TEAM_FROM_M} ? 8 : lego_rowwise_default_wpr(n); }}", ""]
+          f"{rowwise.MAX_N_SMALL_TEAMS} && m >= {ROWWISE_WIDE_TEAM_FROM_M} ? 8 : n > 2048 && n <= 4096 && m > 2048 && m <= 4096 ? 2 "
+          ": lego_rowwise_default_wpr(n); }", ""]
     h += ["unsigned lego_layernorm_bwd_groups(int M, int N);", "unsigned lego_layernorm_bwd_f32_groups(int M, int N);",
           "unsigned lego_layernorm_bwd_bf16_groups(int M, int N);",
           "hipError_t lego_layernorm_bwd_f32_launch(const void*, const void*, const void*, const float*, const float*, "

@@ -159,7 +159,8 @@ def _assert_layernorm_forward(y, x, w, b, eps=1e-5):
 
 @pytest.mark.parametrize("wpr", [None, 1, 2, 4, 8])
 @pytest.mark.parametrize("M,N", [(7, 8), (33, 520), (64, 1024), (5, 2048), (129, 4096), (16, 8192), (3, 16384),
-                                 (4100, 8200)])     # tall and long: the default takes teams of eight waves
+                                 (4100, 8200),      # tall and long: the default takes teams of eight waves
+                                 (2500, 3080)])     # one round of workgroups: the default takes teams of two
 def test_softmax_matches_oracle(ops, M, N, wpr):
     print(f"softmax {M}x{N} wpr={wpr}", flush=True)
     if wpr is not None and N > min(8192 * wpr, 16384):
@@ -299,7 +300,8 @@ def test_layernorm_fp32_long_rows_through_the_c_abi(ops, N):
 # 1151 and 4100 rows with eight waves: workgroups that stage gamma and beta in LDS and walk two to nine rows each
 # 600 and 515 rows of more than 16384 elements: the same walk with sixteen waves, one row across 1024 lanes
 @pytest.mark.parametrize("M,N", [(7, 8), (33, 520), (64, 1024), (129, 4096), (1151, 8192), (3, 16384), (4100, 8200),
-                                 (1030, 16384), (600, 32768), (515, 20488), (511, 32768)])
+                                 (1030, 16384), (600, 32768), (515, 20488), (511, 32768),
+                                 (2500, 3080)])     # one round of workgroups: the default takes teams of two waves
 def test_layernorm_matches_oracle(ops, M, N, wpr):
     print(f"layernorm {M}x{N} wpr={wpr}", flush=True)
     if wpr is not None and N > min(8192 * wpr, 16384):
