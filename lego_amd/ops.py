@@ -107,6 +107,9 @@ def layer_norm_fwd(x, weight, bias, eps=1e-5, waves_per_row: int | None = None):
     return (y if x.dim() == 2 else y.view(x.shape)), mean, rstd
 
 
+_bwd_workspace = {}      # (element tag, M, N) -> bytes of fp32 partial sums
+
+
 def layer_norm_bwd(dy, x, weight, mean, rstd):
     """LayerNorm backward; returns ``(dx, dw, db)``.  fp16, bf16 or fp32 tensors, rows of up to 32768 elements."""
     if x.dtype not in _ROW_TAG:
@@ -124,11 +127,16 @@ def layer_norm_bwd(dy, x, weight, mean, rstd):
         _check(stat, torch.float32, name, ndim=1)       # the forward pass's fp32 statistics, one per row
         if stat.shape[0] != M or stat.device != x.device:
             raise ValueError(f"{name} must hold one float32 per row of x, on its device")
-    need = ctypes.c_ulonglong(0)
-    runtime.call("lego_hip_layernorm_bwd_workspace_bytes" if tag == "f16" else f"lego_hip_layernorm_bwd_{tag}_workspace_bytes",
-                 M, N, ctypes.byref(need))
+    need = _bwd_workspace.get((tag, M, N))
+    if need is None:      # asked once per shape: the answer is a function of the shape alone
+        size = ctypes.c_ulonglong(0)
+        runtime.call("lego_hip_layernorm_bwd_workspace_bytes" if tag == "f16" else f"lego_hip_layernorm_bwd_{tag}_workspace_bytes",
+                     M, N, ctypes.byref(size))
+        if len(_bwd_workspace) >= 4096:
+            _bwd_workspace.clear()
+        need = _bwd_workspace[(tag, M, N)] = size.value
     # like the reference's wrapper, which allocates its partial buffers with torch (layernorm.py:381-383)
-    workspace = torch.empty(need.value // 4, dtype=torch.float32, device=x.device)
+    workspace = torch.empty(need // 4, dtype=torch.float32, device=x.device)
     dx = torch.empty_like(x_arg)
     dw = torch.empty((N,), dtype=weight.dtype, device=x.device)
     db = torch.empty((N,), dtype=weight.dtype, device=x.device)
@@ -176,6 +184,9 @@ def _operand(t, name):
     raise ValueError(f"{name} must be contiguous or the transpose of a contiguous tensor")
 
 
+_gemm_workspace = {}      # (M, N, K) -> bytes of workspace that lego_hip_gemm_ex_ws uses
+
+
 def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "", out_dtype=torch.float16) -> torch.Tensor:
     """``act(a @ b)`` for fp16, bf16 or 8-bit floating-point operands of any shape, each row-major or
     column-major (a ``.T`` view), fp32 accumulation, row-major fp16 result: the reference's ``matmul``
@@ -206,10 +217,15 @@ def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "", out_dtype=tor
     c = torch.empty((M, N), device=a.device, dtype=out_dtype)
     # products of few tiles (a skinny operand, a long K) are split along K when there is room for the partial sums;
     # shapes whose operand rows are not whole 16-byte chunks run on zero-padded copies in the workspace
-    need = ctypes.c_ulonglong(0)
-    runtime.call("lego_hip_gemm_workspace_bytes", M, N, K, ctypes.byref(need))
-    if need.value:
-        workspace = torch.empty(need.value // 4, dtype=torch.float32, device=a.device)
+    need = _gemm_workspace.get((M, N, K))
+    if need is None:      # asked once per shape
+        size = ctypes.c_ulonglong(0)
+        runtime.call("lego_hip_gemm_workspace_bytes", M, N, K, ctypes.byref(size))
+        if len(_gemm_workspace) >= 4096:
+            _gemm_workspace.clear()
+        need = _gemm_workspace[(M, N, K)] = size.value
+    if need:
+        workspace = torch.empty(need // 4, dtype=torch.float32, device=a.device)
         element = 0 if a.dtype == torch.float16 else 4 if out_dtype == torch.float16 else 1
         runtime.call("lego_hip_gemm_ex_ws", element, _ptr(a_store), _ptr(b_store), _ptr(c), M, N, K, ta, tb,
                      1 if activation else 0, _ptr(workspace), need, _stream())
