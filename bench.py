@@ -254,6 +254,53 @@ def main():
                                                          frac_hbm=3 * m3 * n3 * 2 / ms_b / 1e6 / HBM_PEAK_GBS,
                                                          bytes=3 * m3 * n3 * 2, note="cache-resident buffers")
             del dy3, dx3, ws
+            # rows of any length: 8191 elements (the rows of a workgroup start alike and split at the same columns) and
+            # a transpose of odd sides (16-byte accesses at any element); rotating inputs
+            mr, nr = 16386, 8191
+            gr = gen(7)
+            xr = [(2.0 * torch.randn(mr, nr, generator=gr)).half().to(dev) for _ in range(3)]
+            dyr = (0.1 * torch.randn(mr, nr, generator=gr)).half().to(dev)
+            wr = (1 + 0.1 * torch.randn(nr, generator=gr)).half().to(dev)
+            br = (0.1 * torch.randn(nr, generator=gr)).half().to(dev)
+            yr, dxr = torch.empty_like(xr[0]), torch.empty_like(xr[0])
+            dwr, dbr = torch.empty_like(wr), torch.empty_like(br)
+            meanr, rstdr = torch.empty(mr, device=dev), torch.empty(mr, device=dev)
+            runtime.call("lego_hip_layernorm_bwd_workspace_bytes", mr, nr, ctypes.byref(need))
+            wsr = torch.empty(need.value // 4, device=dev)
+            turn = [0]
+
+            def lnr():
+                turn[0] = (turn[0] + 1) % 3
+                runtime.call("lego_hip_layernorm_fwd_f16", p(xr[turn[0]]), p(yr), p(wr), p(br), p(meanr), p(rstdr), mr, nr, 1e-5, stream)
+
+            def smr():
+                turn[0] = (turn[0] + 1) % 3
+                runtime.call("lego_hip_softmax_f16", p(xr[turn[0]]), p(yr), mr, nr, stream)
+
+            def lnbr():
+                turn[0] = (turn[0] + 1) % 3
+                runtime.call("lego_hip_layernorm_bwd_f16", p(dyr), p(xr[turn[0]]), p(wr), p(meanr), p(rstdr), p(dxr), p(dwr),
+                             p(dbr), p(wsr), need, mr, nr, stream)
+            for name, fn, passes in (("next_softmax_f16_16386x8191_any_length", smr, 2),
+                                     ("next_layernorm_fwd_f16_16386x8191_any_length", lnr, 2),
+                                     ("next_layernorm_bwd_f16_16386x8191_any_length", lnbr, 3)):
+                ms_r = timed(fn)
+                kernels[name] = dict(ms=ms_r, gbs=passes * mr * nr * 2 / ms_r / 1e6,
+                                     frac_hbm=passes * mr * nr * 2 / ms_r / 1e6 / HBM_PEAK_GBS)
+            del xr, dyr, yr, dxr, wsr
+            for rows_t, cols_t in ((9999, 10001),):
+                xt = [torch.randn(rows_t, cols_t, generator=gr).half().to(dev) for _ in range(3)]
+                ot = torch.empty(cols_t, rows_t, dtype=torch.half, device=dev)
+
+                def trr():
+                    turn[0] = (turn[0] + 1) % 3
+                    runtime.call("lego_hip_transpose_f16", p(xt[turn[0]]), p(ot), rows_t, cols_t, stream)
+                trr()
+                assert torch.equal(ot, xt[turn[0]].t())
+                ms_t = timed(trr)
+                kernels[f"next_transpose_f16_{rows_t}x{cols_t}_any_shape"] = dict(
+                    ms=ms_t, gbs=2 * rows_t * cols_t * 2 / ms_t / 1e6, frac_hbm=2 * rows_t * cols_t * 2 / ms_t / 1e6 / HBM_PEAK_GBS)
+                del xt, ot
         del x3, y3
 
     # ---- C4: fp16 GEMM 8192^3 ----------------------------------------------------------------------
