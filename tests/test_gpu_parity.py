@@ -248,13 +248,12 @@ def test_layernorm_ragged_and_fp32(ops, dtype, M, N):
 
 
 @pytest.mark.parametrize("M,N", [(24600, 8191), (201500, 1001)])
-def test_rows_of_any_length_results_past_the_cache(ops, M, N):
-    """fp16 results of more than 384 MiB: the kernels for rows of any length store them with non-temporal
-    stores (another instantiation), the walking kernels in launches of at most 16 rows per team.  At this size:
+def test_rows_of_any_length_in_several_launches(ops, M, N):
+    """Tall matrices of rows of any length: the walking kernels run in launches of at most 16 rows per team, one
+    after the other.  At this size:
     row sums of the softmax, the statistics against torch on the GPU, and the first and last rows (the ends of
     the first and of the last launch) against the oracle."""
     print(f"rows of any length, large result {M}x{N}", flush=True)
-    assert M * N * 2 > 384 << 20
     g = _gen(61)
     xd = (2.0 * torch.randn(M, N, generator=g, dtype=torch.float32)).half().cuda()
     w = (1 + 0.1 * torch.randn(N, generator=g)).half()
