@@ -179,6 +179,7 @@ int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream)
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 8)   // ragged rows
     return ok_or((N <= 128 ? lego_softmax_f16s_l16_launch : N <= 256 ? lego_softmax_f16s_l32_launch
+                  : lego_rowwise_f16_wpr(M, N) == 8 ? lego_softmax_f16s_w8_launch
                   : long_row ? lego_softmax_f16s_w16_launch : lego_rowwise_default_wpr(N) == 1 ? lego_softmax_f16s_w1_launch
                                                                                            : lego_softmax_f16s_w4_launch)(
         x, y, M, N, as_stream(stream)));
@@ -230,6 +231,7 @@ int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 8)   // ragged rows
     return ok_or((N <= 128 ? lego_layernorm_fwd_f16s_l16_launch : N <= 256 ? lego_layernorm_fwd_f16s_l32_launch
+                  : lego_rowwise_f16_wpr(M, N) == 8 ? lego_layernorm_fwd_f16s_w8_launch
                   : long_row ? lego_layernorm_fwd_f16s_w16_launch : lego_rowwise_default_wpr(N) == 1 ? lego_layernorm_fwd_f16s_w1_launch
                                                                                                  : lego_layernorm_fwd_f16s_w4_launch)(
         x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));
@@ -264,6 +266,7 @@ int lego_hip_softmax_bf16(const void* x, void* y, int M, int N, void* stream)
   const int wpr = lego_rowwise_default_wpr(N);
   if (N % 8)   // ragged rows
     return ok_or((N <= 128 ? lego_softmax_bf16s_l16_launch : N <= 256 ? lego_softmax_bf16s_l32_launch
+                  : lego_rowwise_f16_wpr(M, N) == 8 ? lego_softmax_bf16s_w8_launch
                   : wpr == 16 ? lego_softmax_bf16s_w16_launch : wpr == 1 ? lego_softmax_bf16s_w1_launch
                                                                        : lego_softmax_bf16s_w4_launch)(x, y, M, N, as_stream(stream)));
   if (N <= 256) return ok_or((N <= 128 ? lego_softmax_bf16_l16_launch : lego_softmax_bf16_l32_launch)(x, y, M, N, as_stream(stream)));
@@ -280,6 +283,7 @@ int lego_hip_layernorm_fwd_bf16(const void* x, void* y, const void* w, const voi
   const int wpr = lego_rowwise_default_wpr(N);
   if (N % 8)   // ragged rows
     return ok_or((N <= 128 ? lego_layernorm_fwd_bf16s_l16_launch : N <= 256 ? lego_layernorm_fwd_bf16s_l32_launch
+                  : lego_rowwise_f16_wpr(M, N) == 8 ? lego_layernorm_fwd_bf16s_w8_launch
                   : wpr == 16 ? lego_layernorm_fwd_bf16s_w16_launch : wpr == 1 ? lego_layernorm_fwd_bf16s_w1_launch
                                                                              : lego_layernorm_fwd_bf16s_w4_launch)(
         x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));

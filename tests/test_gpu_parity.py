@@ -208,7 +208,9 @@ def test_softmax_reference_test_shape_fp32(ops):
                                  (8300, 781), (8195, 250), (8200, 1001), (2050, 4099), (2049, 8191), (2300, 2050),
                                  (1030, 12001), (1100, 16383), (515, 20001), (600, 32767),
                                  # tall, rows of 12-32 KiB: teams of eight waves in fp32 as well
-                                 (4100, 4096), (4097, 8192), (4096, 3076)])
+                                 (4100, 4096), (4097, 8192), (4096, 3076),
+                                 # ... and for 16-bit rows of any length
+                                 (4100, 8191), (4097, 12001)])
 def test_softmax_ragged_and_fp32(ops, dtype, M, N):
     print(f"softmax {dtype} {M}x{N}", flush=True)
     x = (2.0 * torch.randn(M, N, generator=_gen(2))).to(dtype)
@@ -224,7 +226,9 @@ def test_softmax_ragged_and_fp32(ops, dtype, M, N):
                                  (8300, 781), (8195, 250), (8200, 1001), (2050, 4099), (2049, 8191), (2300, 2050),
                                  (515, 20001), (600, 32767), (1030, 12001), (1100, 16383), (4100, 3001),
                                  # tall, rows of 12-32 KiB: teams of eight waves in fp32 as well (gamma and beta in LDS)
-                                 (4100, 4096), (4097, 8192), (4096, 3076)])
+                                 (4100, 4096), (4097, 8192), (4096, 3076),
+                                 # ... and for 16-bit rows of any length
+                                 (4100, 8191), (4097, 12001)])
 def test_layernorm_ragged_and_fp32(ops, dtype, M, N):
     print(f"layernorm {dtype} {M}x{N}", flush=True)
     if N * torch.empty((), dtype=dtype).element_size() > 65536:
@@ -451,7 +455,7 @@ def test_short_rows_share_a_wave(ops, dtype, M, N):
 
 
 @pytest.mark.parametrize("M,N", [(5, 8), (9, 781), (33, 2048), (64, 8192), (3, 8191), (4, 20000), (2, 32768), (2, 50257),
-                                 (4100, 8200)])      # tall and long: teams of eight waves
+                                 (4100, 8200), (4100, 8191)])      # tall and long: teams of eight waves
 def test_softmax_bfloat16(ops, M, N):
     print(f"softmax bf16 {M}x{N}", flush=True)
     x = (2.0 * torch.randn(M, N, generator=_gen(30))).bfloat16()
@@ -464,7 +468,7 @@ def test_softmax_bfloat16(ops, M, N):
 
 @pytest.mark.parametrize("M,N", [(5, 8), (9, 781), (33, 2048), (64, 8192), (3, 8191), (4, 20000), (2, 32768),
                                  (4100, 8200), (530, 24576),    # tall and long: gamma and beta staged in LDS
-                                 (1100, 781), (530, 8191), (260, 16383)])
+                                 (1100, 781), (530, 8191), (260, 16383), (4100, 8191)])
 def test_layernorm_bfloat16_forward_and_backward(ops, M, N):
     """bfloat16 tensors through the autograd wrapper, against fp32 autograd on the CPU."""
     from lego_amd.ops import lego_layer_norm
