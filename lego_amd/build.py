@@ -45,7 +45,7 @@ TRANSPOSE = {
 # (element type, vectorised, waves per row): 16-byte accesses need N % (16/size) == 0; the
 # element-per-access kernels ("s") take any N
 ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f16", True, 8), ("f32", True, 1), ("f32", True, 4), ("f32", True, 8),
-           ("f16", False, 1), ("f32", False, 1), ("f16", False, 4), ("f32", False, 4), ("f16", False, 8), ("bf16", False, 8),
+           ("f16", False, 1), ("f32", False, 1), ("f16", False, 4), ("f32", False, 4), ("f16", False, 8), ("bf16", False, 8), ("f32", False, 8),
            ("f16", True, 16), ("f32", True, 16), ("f16", False, 16), ("f32", False, 16),
            ("bf16", True, 1), ("bf16", True, 4), ("bf16", True, 8), ("bf16", True, 16), ("bf16", False, 1), ("bf16", False, 4),
            ("bf16", False, 16)]
@@ -55,7 +55,7 @@ ROWWISE_SHORT = [(d, lanes, vec) for d in ("f16", "bf16", "f32") for lanes in (1
 ROWWISE_STREAM_WGS = {("f16", True, 8): 512, ("bf16", True, 8): 512, ("f32", True, 8): 512, ("f16", True, 16): 256, ("bf16", True, 16): 256,
                       # rows of any length: a team's rows must start alike, so the count times the teams per workgroup is a multiple of 8
                       ("f16", False, 1): 1024, ("f16", False, 4): 1024, ("f16", False, 16): 256,
-                      ("f16", False, 8): 512, ("bf16", False, 8): 512,
+                      ("f16", False, 8): 512, ("bf16", False, 8): 512, ("f32", False, 8): 512,
                       ("bf16", False, 1): 1024, ("bf16", False, 4): 1024, ("bf16", False, 16): 256,
                       ("f32", False, 1): 1024, ("f32", False, 4): 1024, ("f32", False, 16): 256}
 ROWWISE_DEFAULT_WAVES = 4

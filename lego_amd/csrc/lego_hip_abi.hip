@@ -193,6 +193,7 @@ int lego_hip_softmax_f32(const void* x, void* y, int M, int N, void* stream)
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 4)   // ragged rows
     return ok_or((N <= 64 ? lego_softmax_f32s_l16_launch : N <= 128 ? lego_softmax_f32s_l32_launch
+                  : lego_rowwise_f16_wpr(M, 2 * N) == 8 ? lego_softmax_f32s_w8_launch
                   : long_row ? lego_softmax_f32s_w16_launch : N <= 1024 ? lego_softmax_f32s_w1_launch
                                                                       : lego_softmax_f32s_w4_launch)(x, y, M, N, as_stream(stream)));
   if (N <= 1024)   // rows of at most 16 or 32 vectors: several rows per wave
@@ -246,6 +247,7 @@ int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
   if (N % 4)   // ragged rows
     return ok_or((N <= 64 ? lego_layernorm_fwd_f32s_l16_launch : N <= 128 ? lego_layernorm_fwd_f32s_l32_launch
+                  : lego_rowwise_f16_wpr(M, 2 * N) == 8 ? lego_layernorm_fwd_f32s_w8_launch
                   : long_row ? lego_layernorm_fwd_f32s_w16_launch : N <= 1024 ? lego_layernorm_fwd_f32s_w1_launch
                                                                             : lego_layernorm_fwd_f32s_w4_launch)(
         x, y, w, b, mean, rstd, M, N, eps, as_stream(stream)));

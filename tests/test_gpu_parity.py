@@ -210,7 +210,7 @@ def test_softmax_reference_test_shape_fp32(ops):
                                  # tall, rows of 12-32 KiB: teams of eight waves in fp32 as well
                                  (4100, 4096), (4097, 8192), (4096, 3076),
                                  # ... and for 16-bit rows of any length
-                                 (4100, 8191), (4097, 12001)])
+                                 (4100, 8191), (4097, 12001), (4100, 4099)])
 def test_softmax_ragged_and_fp32(ops, dtype, M, N):
     print(f"softmax {dtype} {M}x{N}", flush=True)
     x = (2.0 * torch.randn(M, N, generator=_gen(2))).to(dtype)
@@ -228,7 +228,7 @@ def test_softmax_ragged_and_fp32(ops, dtype, M, N):
                                  # tall, rows of 12-32 KiB: teams of eight waves in fp32 as well (gamma and beta in LDS)
                                  (4100, 4096), (4097, 8192), (4096, 3076),
                                  # ... and for 16-bit rows of any length
-                                 (4100, 8191), (4097, 12001)])
+                                 (4100, 8191), (4097, 12001), (4100, 4099)])
 def test_layernorm_ragged_and_fp32(ops, dtype, M, N):
     print(f"layernorm {dtype} {M}x{N}", flush=True)
     if N * torch.empty((), dtype=dtype).element_size() > 65536:
