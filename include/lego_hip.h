@@ -29,7 +29,7 @@ int lego_hip_abi_version(void);
  * mlir_generated/transpose/transpose_smem_4096.mlir:24-97), which have no callable entry.
  * Any shape; rows and cols in whole 16-byte vectors (multiples of 8 for 2-byte, of 4 for 4-byte
  * elements) take the 16-byte-per-lane kernels, without edge tests when they are whole tiles;
- * other shapes the same kernels with 16-byte accesses at any element (about two thirds as fast), small
+ * other shapes the same kernels with 16-byte accesses at any element (about two thirds as fast), tiny
  * ones a kernel that moves one element per access.  _f32 moves 4-byte
  * elements, _f16 2-byte elements, whatever their type. */
 int lego_hip_transpose_f32(const void* in, void* out, int rows, int cols, void* stream);

@@ -33,14 +33,16 @@ TRANSPOSE = {
             dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag"),
             dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag"),
             dict(dtype="f32", tile=(32, 32), group=(2, 4), order="col", edge=True, xcd=True),
-            dict(dtype="f32", tile=(32, 32), group=(4, 2), order="col", edge=True, ragged=True, xcd=True)],
+            dict(dtype="f32", tile=(32, 32), group=(4, 2), order="col", edge=True, ragged=True, xcd=True),
+            dict(dtype="f32", tile=(32, 32), group=(2, 2), order="col", edge=True, ragged=True, xcd=True)],
     "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 128, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 64, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 32, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag"),
             dict(dtype="f16", tile=(64, 64), group=(1, 1), order="diag"),
             dict(dtype="f16", tile=(64, 64), group=(2, 2), order="col", edge=True, xcd=True),
-            dict(dtype="f16", tile=(64, 64), group=(2, 2), order="col", edge=True, ragged=True, xcd=True)],
+            dict(dtype="f16", tile=(64, 64), group=(2, 2), order="col", edge=True, ragged=True, xcd=True),
+            dict(dtype="f16", tile=(64, 64), group=(1, 1), order="col", edge=True, ragged=True, xcd=True)],
 }
 # (element type, vectorised, waves per row): 16-byte accesses need N % (16/size) == 0; the
 # element-per-access kernels ("s") take any N
@@ -85,7 +87,10 @@ def collect():
             if cfg.get("ragged"):     # any shape with at least one whole vector per row of both matrices
                 meta["row_multiple"] = meta["col_multiple"] = 1
                 meta["min_side"] = vec
-                meta["min_elements"] = 256 * meta["SR"] * meta["SC"]     # a macro tile per CU; smaller matrices take 64x64 tiles
+                # 64x64 tiles up to 64 Mi elements (fp16 4099 x 4101: 3.9 against 3.1 TB/s with 128x128 tiles, 6001 x 6003 3.5
+                # against 3.3), the larger tile above (9999 x 10001: 3.5 against 3.4); matrices of under 16 Ki elements
+                # go one element per access
+                meta["min_elements"] = (64 << 20) if meta["SR"] * meta["SC"] > 64 * 64 else (16 << 10)
             unit.filename = meta["kernel"].replace("lego_", "", 1) + ".hip"
             units.append(unit)
             tmeta.setdefault(dtype, []).append(meta)

@@ -87,15 +87,16 @@ def test_transpose_moves_bits_of_any_2_or_4_byte_type(ops, dtype):
                                              (torch.float16, 1000, 777), (torch.float16, 777, 1000), (torch.float16, 7, 300),
                                              (torch.float32, 5, 7), (torch.float32, 1001, 999), (torch.float32, 130, 257),
                                              (torch.float32, 2051, 1033), (torch.float32, 516, 1001), (torch.float32, 1001, 516),
-                                             # ... from a macro tile per CU on (smaller matrices take the 64x64 tiles)
                                              (torch.float16, 2055, 2061), (torch.float16, 15, 300001), (torch.float16, 300001, 15),
                                              (torch.float16, 4100, 1031), (torch.float16, 1031, 4100),
                                              (torch.float32, 1449, 1451), (torch.float32, 5, 500001), (torch.float32, 500001, 5),
-                                             (torch.float32, 2052, 1031)])
+                                             (torch.float32, 2052, 1031),
+                                             # the larger macro tile, from 64 Mi elements on
+                                             (torch.float16, 8200, 8201), (torch.float32, 8197, 8199)])
 def test_transpose_of_any_shape(ops, dtype, rows, cols):
     """Shapes no tiling divides: in whole 16-byte vectors both ways they take the wide tile with edge
-    tests, otherwise the same tile with vectors at any element, and the one-element-per-access kernel when a
-    side is shorter than a vector."""
+    tests, otherwise 64x64 tiles (a larger tile from 64 Mi elements on) with vectors at any element, and the
+    one-element-per-access kernel when a side is shorter than a vector or the matrix is tiny."""
     print(f"transpose (any shape) {dtype} {rows}x{cols}", flush=True)
     x = (torch.rand(rows, cols, generator=_gen(4)) * 2 - 1).to(dtype)
     want = ok.transpose(x, 1, 1)
