@@ -84,6 +84,9 @@ def collect():
             if cfg.get("edge"):
                 vec = 4 if dtype == "f32" else 8
                 meta["row_multiple"] = meta["col_multiple"] = vec
+                # smaller matrices have too few of these macro tiles: the 64x64 ones of the any-shape kernels are ahead up
+                # to about 32 Mi elements (fp16 2056^2 3.2 against 2.3 TB/s, 4104^2 4.2 / 3.8; 6152^2 3.7 / 4.0)
+                meta["min_elements"] = 32 << 20
             if cfg.get("ragged"):     # any shape with at least one whole vector per row of both matrices
                 meta["row_multiple"] = meta["col_multiple"] = 1
                 meta["min_side"] = vec
@@ -133,14 +136,16 @@ def collect():
     for dtype, metas in tmeta.items():
         for m in metas:
             h.append(f"hipError_t {m['kernel']}_launch(const void*, void*, int, int, hipStream_t);")
-        h += [f"// picks the first tiling that divides the shape; any other shape takes the same tiling with vectors at any element and edge tests, a small matrix the one-element-per-access kernel (64x64 tiles)",
+        h += [f"// picks the first tiling that divides the shape; any other shape takes the tiling with vectors at any element and edge tests, a tiny matrix the one-element-per-access kernel",
               f"inline hipError_t lego_transpose_{dtype}_dispatch(const void* in, void* out, int rows, int cols, "
               "hipStream_t stream) {"]
         for m in metas:
             fits = "" if m["max_bytes"] is None else \
                 f" && 2ull * rows * cols * {4 if dtype == 'f32' else 2} <= {m['max_bytes']}ull"
             if m.get("min_side"):
-                fits += f" && rows >= {m['min_side']} && cols >= {m['min_side']} && 1ull * rows * cols >= {m['min_elements']}ull"
+                fits += f" && rows >= {m['min_side']} && cols >= {m['min_side']}"
+            if m.get("min_elements"):
+                fits += f" && 1ull * rows * cols >= {m['min_elements']}ull"
             h.append(f"  if (rows % {m['row_multiple']} == 0 && cols % {m['col_multiple']} == 0{fits}) "
                      f"return {m['kernel']}_launch(in, out, rows, cols, stream);")
         h += [f"  return lego_transpose_any_launch(in, out, rows, cols, {4 if dtype == 'f32' else 2}, stream);", "}", ""]

@@ -92,7 +92,11 @@ def test_transpose_moves_bits_of_any_2_or_4_byte_type(ops, dtype):
                                              (torch.float32, 1449, 1451), (torch.float32, 5, 500001), (torch.float32, 500001, 5),
                                              (torch.float32, 2052, 1031),
                                              # the larger macro tile, from 64 Mi elements on
-                                             (torch.float16, 8200, 8201), (torch.float32, 8197, 8199)])
+                                             (torch.float16, 8200, 8201), (torch.float32, 8197, 8199),
+                                             # whole vectors, from 32 Mi elements on: the wide tile with edge tests, rows
+                                             # in cut and in whole 64-byte blocks (plain and non-temporal stores)
+                                             (torch.float16, 8200, 4104), (torch.float16, 8224, 4128),
+                                             (torch.float32, 8196, 4100), (torch.float32, 8208, 4112)])
 def test_transpose_of_any_shape(ops, dtype, rows, cols):
     """Shapes no tiling divides: in whole 16-byte vectors both ways they take the wide tile with edge
     tests, otherwise 64x64 tiles (a larger tile from 64 Mi elements on) with vectors at any element, and the
