@@ -30,7 +30,7 @@ OBJ_DIR = LIB_DIR / "obj"
 TRANSPOSE = {
     "f32": [dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 64, 8), max_bytes=1536 << 20),
             dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 32, 8), max_bytes=1536 << 20),
-            dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag"),
+            dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag", min_elements=2 << 20),   # smaller: 64x64 tiles
             dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag"),
             dict(dtype="f32", tile=(32, 32), group=(2, 4), order="col", edge=True, xcd=True),
             dict(dtype="f32", tile=(32, 32), group=(4, 2), order="col", edge=True, ragged=True, xcd=True),
@@ -38,7 +38,7 @@ TRANSPOSE = {
     "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 128, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 64, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 32, 8)),
-            dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag"),
+            dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag", min_elements=2 << 20),   # smaller: 64x64 tiles
             dict(dtype="f16", tile=(64, 64), group=(1, 1), order="diag"),
             dict(dtype="f16", tile=(64, 64), group=(2, 2), order="col", edge=True, xcd=True),
             dict(dtype="f16", tile=(64, 64), group=(2, 2), order="col", edge=True, ragged=True, xcd=True),
@@ -79,8 +79,11 @@ def collect():
         for cfg in configs:
             cfg = dict(cfg)
             max_bytes = cfg.pop("max_bytes", None)   # only for matrices that fit the last-level cache
+            min_elements = cfg.pop("min_elements", None)
             unit, meta = transpose.emit(**cfg, suffix="")
             meta["max_bytes"] = max_bytes
+            if min_elements:
+                meta["min_elements"] = min_elements
             if cfg.get("edge"):
                 vec = 4 if dtype == "f32" else 8
                 meta["row_multiple"] = meta["col_multiple"] = vec

@@ -31,6 +31,7 @@ def _gen(seed):
     (torch.float16, 8192, 2048),                    # one window of the windowed tile order
     (torch.float16, 4096, 6144), (torch.float16, 12288, 2048),    # windows of 64 x 8 macro tiles: one, and three by one
     (torch.float16, 2048, 4096), (torch.float16, 6144, 2048),     # windows of 32 x 8: one by two, three by one
+    (torch.float16, 1088, 2304), (torch.float32, 1056, 2304),     # the wide tiles in skewed order (from 2 Mi elements on)
 ])
 def test_transpose_matches_oracle(ops, dtype, rows, cols):
     print(f"transpose {dtype} {rows}x{cols}", flush=True)
