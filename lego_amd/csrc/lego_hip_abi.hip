@@ -387,6 +387,17 @@ struct GemmKernels {
 // Fewer 256 x 256 tiles than this and the 128 x 128 kernel, with four times as many workgroups,
 // keeps more of the 256 CUs busy than its higher LDS traffic per flop costs.
 constexpr long kSmallTileBelow = 129;
+// The same for larger products whose 256 x 256 tiles leave the last round of workgroups mostly empty: the share of
+// workgroup slots that do work, over whole rounds of 256 (512 for the small tile, which runs at about 0.8 of the
+// large tile's rate), decides.  4608^3, 324 tiles in two rounds: 0.98 -> 1.02 PFLOP/s; 5120^3 and 6144^3 stay.
+inline bool small_tiles_fill_better(int M, int N, long tiles)
+{
+  if (tiles < kSmallTileBelow) return true;
+  const long small = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
+  const double fill_big = static_cast<double>(tiles) / (256 * ((tiles + 255) / 256));
+  const double fill_small = static_cast<double>(small) / (512 * ((small + 511) / 512));
+  return 0.8 * fill_small > fill_big;
+}
 
 int gemm_ex(const GemmKernels& k, int element, const void* a, const void* b, void* c, int M, int N, int K,
             int trans_a, int trans_b, int activation, void* stream, int bk = LEGO_GEMM_BK, int chunk = 8)
@@ -410,7 +421,7 @@ int gemm_ex(const GemmKernels& k, int element, const void* a, const void* b, voi
   }
   const long tiles = static_cast<long>((M + LEGO_GEMM_BM - 1) / LEGO_GEMM_BM) * ((N + LEGO_GEMM_BN - 1) / LEGO_GEMM_BN);
   const int layout = (trans_a ? 2 : 0) + (trans_b ? 1 : 0);
-  const gemm_launcher* by_layout = tiles < kSmallTileBelow && k.small[layout] != nullptr ? k.small : k.big;
+  const gemm_launcher* by_layout = small_tiles_fill_better(M, N, tiles) && k.small[layout] != nullptr ? k.small : k.big;
   return ok_or(by_layout[layout](a, b, c, M, N, K, activation, as_stream(stream)));
 }
 
