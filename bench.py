@@ -166,6 +166,38 @@ def main():
     kernels["device_copy16_512MiB"] = dict(ms=copy16_ms, gbs=bytes2 / copy16_ms / 1e6,
                                            note="plain 16-byte-per-lane copy kernel of this library (counter calibration)")
 
+    # ---- what the memory delivers here: one-directional streams and copies on rotating 512 MiB buffers ----------
+    # (three pairs in turn, so that nothing is served by the 256 MB last-level cache).  A kernel that reads and writes
+    # every byte once spends half its bytes in each direction: it cannot pass 1 / (0.5 / read + 0.5 / write).
+    probe_bytes = 512 << 20
+    pin = [x2.view(-1)[:probe_bytes // 2]] + [torch.randn(probe_bytes // 2, device=dev).half() for _ in range(2)]
+    pout = [y2.view(-1)[:probe_bytes // 2]] + [torch.empty(probe_bytes // 2, dtype=torch.half, device=dev) for _ in range(2)]
+    turn_p = [0]
+
+    def probe(mode, vectors):
+        def fn():
+            turn_p[0] = (turn_p[0] + 1) % 3
+            runtime.call("lego_hip_hbm_probe", p(pin[turn_p[0]]), p(pout[turn_p[0]]), ctypes.c_ulonglong(probe_bytes),
+                         mode, vectors, stream)
+        return fn
+    ceiling = {}
+    for label, mode, vectors, moved in (("read_only_16KiB_per_wg", 0, 4, 1), ("write_only_16KiB_per_wg", 1, 4, 1),
+                                        ("read_only_4KiB_per_wg", 0, 1, 1), ("write_only_4KiB_per_wg", 1, 1, 1),
+                                        ("copy_16KiB_per_wg", 2, 4, 2), ("copy_4KiB_per_wg", 2, 1, 2)):
+        ms_p = timed(probe(mode, vectors))
+        ceiling[label] = dict(ms=ms_p, gbs=moved * probe_bytes / ms_p / 1e6)
+    read_gbs = max(ceiling["read_only_16KiB_per_wg"]["gbs"], ceiling["read_only_4KiB_per_wg"]["gbs"])
+    write_gbs = max(ceiling["write_only_16KiB_per_wg"]["gbs"], ceiling["write_only_4KiB_per_wg"]["gbs"])
+    achievable = 1.0 / (0.5 / read_gbs + 0.5 / write_gbs)
+    ceiling["read_plus_write_bound_gbs"] = achievable
+    ceiling["note"] = ("non-temporal 16-byte accesses, 256 lanes per workgroup, 1 or 4 vectors per lane; three rotating pairs "
+                       "of 512 MiB buffers; read_plus_write_bound = 1 / (0.5 / best read-only + 0.5 / best write-only): the "
+                       "rate a kernel that reads and writes every byte once cannot pass on this part")
+    kernels["hbm_ceiling"] = ceiling
+    kernels["c2_transpose_f16_16384"].update(achievable_gbs=achievable, frac_of_achievable=gbs2 / achievable)
+    c2()      # y2 holds the transpose again (the probes wrote into it)
+    del pin, pout
+
     # ---- C1: fp32 4096^2 transpose ---------------------------------------------------------
     if want("c1"):
         n1 = 4096
@@ -179,6 +211,7 @@ def main():
                        1 << 30, b1)
         kernels["c1_transpose_f32_4096"] = dict(ms_hot=hot, gbs_hot=b1 / hot / 1e6, ms=rot, gbs=b1 / rot / 1e6,
                                                 frac_hbm=b1 / rot / 1e6 / HBM_PEAK_GBS, bytes=b1,
+                                                achievable_gbs=achievable, frac_of_achievable=b1 / rot / 1e6 / achievable,
                                                 parity="bit-exact",
                                                 note="gbs = rotating buffers (1 GiB pool); gbs_hot = cache resident")
         if not ns.skip_cpu:
@@ -227,6 +260,7 @@ def main():
             rot = rotating(mk, fn, 1 << 30, by3)
             kernels[name] = dict(ms_hot=hot, gbs_hot=by3 / hot / 1e6, ms=rot, gbs=by3 / rot / 1e6,
                                  frac_hbm=by3 / rot / 1e6 / HBM_PEAK_GBS, bytes=by3, max_abs_err_vs_fp32=err,
+                                 achievable_gbs=achievable, frac_of_achievable=by3 / rot / 1e6 / achievable,
                                  note="gbs = rotating buffers (1 GiB pool); gbs_hot = cache resident; "
                                       "x ~ N(0, sigma=2)")
         if not ns.skip_cpu:
@@ -550,6 +584,9 @@ def main():
                                "staging, inputs N(0,1) seed 1"},
         "roofline": {"bound": "hbm", "achieved": gbs2, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs2 / HBM_PEAK_GBS, "traffic": headline_traffic_bytes(),
+                     "achievable": achievable, "frac_of_achievable": gbs2 / achievable,
+                     "achievable_note": "1 / (0.5 / read-only + 0.5 / write-only) of this run's one-directional "
+                                        "streams (kernels.hbm_ceiling)",
                      "kernel": HEADLINE_KERNEL, "algorithmic_bytes_per_launch": bytes2},
         "cpu_baseline": cpu,
         "kernels": kernels,

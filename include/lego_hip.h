@@ -195,8 +195,10 @@ int lego_hip_lud_f32_plan(int n, int* records, int capacity, int* count);
 int lego_hip_nw_i32(const int* reference, int* matrix, int n, int penalty, void* stream);
 
 /* groups independent GEMMs in one launch.  a, b, c are HOST arrays of `groups` device
- * pointers; sizes3 is a HOST array of groups*3 ints (M, N, K per problem).  At most 64
- * groups.  One launch when every N and K is a multiple of 8 and every base 16-byte aligned (any M;
+ * pointers; sizes3 is a HOST array of groups*3 ints (M, N, K per problem).  Any number of
+ * groups: one launch carries up to 64 problems (their pointers and sizes travel as kernel arguments), a
+ * call with more is enqueued as runs of 64 in order of decreasing K, one launch after the other on
+ * `stream`.  One launch per run when every N and K is a multiple of 8 and every base 16-byte aligned (any M;
  * ragged tiles and last k-tiles are masked); otherwise one launch per problem, as lego_hip_gemm_f16
  * would take it.  Replaces
  * lego_group_gemm_fn(group_A, group_B) (reference:
@@ -208,7 +210,7 @@ int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* 
 /* What lego_hip_grouped_gemm_f16 launches for these sizes, without touching a device: plan3[0] = tile
  * size (256: 256 x 256 tiles, or 128: 128 x 128 tiles), plan3[1] = number of 256 x 256 tiles of all
  * problems, plan3[2] = how many of them, the last ones of the launch order, are computed as two
- * 128 x 256 halves by two workgroups.  No counterpart in the reference (its kernel walks whole tiles
+ * 128 x 256 halves by two workgroups.  At most 64 groups (one launch).  No counterpart in the reference (its kernel walks whole tiles
  * only, grouped_gemm.py:61-116); it is there so that the launch can be checked on the host. */
 int lego_hip_grouped_gemm_f16_plan(const int* sizes3, int groups, int* plan3);
 /* Tuning entry point: lego_hip_grouped_gemm_f16 with the launch chosen by the caller: split_tiles >= 0
@@ -232,6 +234,17 @@ int lego_hip_copy16(const void* in, void* out, unsigned long long bytes, void* s
  * the bandwidth a kernel that reads and writes every byte once can reach on this part.
  * bytes a multiple of 16384. */
 int lego_hip_copy16_stream(const void* in, void* out, unsigned long long bytes, void* stream);
+
+/* Measurement aid (no counterpart in the reference): what the memory delivers to a stream in one direction, in
+ * the access shape of lego_hip_copy16_stream -- non-temporal 16-byte accesses, vectors_per_lane (1 or 4) of them
+ * per lane, one contiguous chunk of 4 KiB * vectors_per_lane per workgroup of 256 lanes.
+ *   mode 0: read in[0..bytes) and store next to nothing (a lane's words are folded and compared with a constant;
+ *           a lane that matches, one in 2^32 for random data, stores one vector into the first 4 KiB of out);
+ *           mode 1: write out[0..bytes), in is not read;
+ *   mode 2: out[0..bytes) = in[0..bytes).
+ * bytes a multiple of the chunk.  bench.py times modes 0 and 1 on rotating 512 MiB buffers and derives from them
+ * the rate that a kernel which reads and writes every byte once cannot pass on this part. */
+int lego_hip_hbm_probe(const void* in, void* out, unsigned long long bytes, int mode, int vectors_per_lane, void* stream);
 
 #ifdef __cplusplus
 }

@@ -8,7 +8,11 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <string.h>
+
+#include <algorithm>
 #include <mutex>
+#include <vector>
 
 #include "lego_hip.h"
 #include "generated/launchers.h"
@@ -39,6 +43,42 @@ __global__ void __launch_bounds__(256) lego_copy16_stream_kernel(const u32x4* __
   for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(in + base + u * 256);
 #pragma unroll
   for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(v[u], out + base + u * 256);
+}
+
+// What the memory delivers to one-directional streams, in the access shape of lego_copy16_stream_kernel (V
+// non-temporal 16-byte vectors per lane, a contiguous V*4 KiB chunk per workgroup): a read-only stream whose
+// values are folded into one word and compared with a constant (the loads must depend on the data, or the
+// compiler drops them; a lane whose words happen to fold to the constant stores one vector into the first 4 KiB
+// of `sink`), and a write-only stream of a lane-dependent pattern.
+template <int V>
+__global__ void __launch_bounds__(256) lego_probe_read_kernel(const u32x4* __restrict__ in, u32x4* __restrict__ sink)
+{
+  const size_t base = static_cast<size_t>(blockIdx.x) * (256 * V) + threadIdx.x;
+  u32x4 v[V];
+#pragma unroll
+  for (int u = 0; u < V; ++u) v[u] = __builtin_nontemporal_load(in + base + u * 256);
+  unsigned acc = 0;
+#pragma unroll
+  for (int u = 0; u < V; ++u) acc ^= v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3];
+  if (acc == 0x9e3779b9u) sink[threadIdx.x] = v[0];
+}
+template <int V>
+__global__ void __launch_bounds__(256) lego_probe_write_kernel(u32x4* __restrict__ out)
+{
+  const size_t base = static_cast<size_t>(blockIdx.x) * (256 * V) + threadIdx.x;
+  const u32x4 v = {threadIdx.x, blockIdx.x, 3u, 4u};
+#pragma unroll
+  for (int u = 0; u < V; ++u) __builtin_nontemporal_store(v, out + base + u * 256);
+}
+template <int V>
+__global__ void __launch_bounds__(256) lego_probe_copy_kernel(const u32x4* __restrict__ in, u32x4* __restrict__ out)
+{
+  const size_t base = static_cast<size_t>(blockIdx.x) * (256 * V) + threadIdx.x;
+  u32x4 v[V];
+#pragma unroll
+  for (int u = 0; u < V; ++u) v[u] = __builtin_nontemporal_load(in + base + u * 256);
+#pragma unroll
+  for (int u = 0; u < V; ++u) __builtin_nontemporal_store(v[u], out + base + u * 256);
 }
 
 typedef unsigned u32x4w __attribute__((ext_vector_type(4)));
@@ -665,7 +705,6 @@ double grouped_makespan(const long* count, const double* cost, int batches, long
 // order as two 128 x 256 halves each (kind 0), or the kernel on 128 x 128 tiles (kind 1).
 struct GroupedPlan {
   int kind, tiles, split;
-  int order[LEGO_GROUPED_MAX_GROUPS];       // problems in launch order: decreasing depth, stable
 };
 
 // Costs in units of one k-tile step of a 256 x 256 tile that has its CU to itself (about 1.8 us for
@@ -673,22 +712,26 @@ struct GroupedPlan {
 // 16 steps); a 128 x 256 half-tile takes 19.2 us for 16 steps; a 128 x 128 tile sharing its CU with
 // another one takes 0.66 of a whole tile of the same depth.
 constexpr double kTileOverhead = 1.6, kHalfStep = 0.58, kHalfOverhead = 1.5, kSmallCost = 0.66;
+// Problems per call.  A launch carries its pointers and sizes as kernel arguments, LEGO_GROUPED_MAX_GROUPS problems
+// at most; a call with more is enqueued as several launches (below).
+constexpr int kGroupedMaxProblems = 1 << 20;
 
-GroupedPlan grouped_plan(const int* sizes3, int groups)
+GroupedPlan grouped_plan_uncached(const int* sizes3, int groups)
 {
   GroupedPlan plan;
-  for (int g = 0; g < groups; ++g) plan.order[g] = g;
+  int order[LEGO_GROUPED_MAX_GROUPS];       // problems in launch order: decreasing depth, stable
+  for (int g = 0; g < groups; ++g) order[g] = g;
   for (int i = 1; i < groups; ++i) {
-    const int o = plan.order[i];
+    const int o = order[i];
     int j = i;
-    while (j > 0 && sizes3[3 * plan.order[j - 1] + 2] < sizes3[3 * o + 2]) { plan.order[j] = plan.order[j - 1]; --j; }
-    plan.order[j] = o;
+    while (j > 0 && sizes3[3 * order[j - 1] + 2] < sizes3[3 * o + 2]) { order[j] = order[j - 1]; --j; }
+    order[j] = o;
   }
   long big[LEGO_GROUPED_MAX_GROUPS], small[LEGO_GROUPED_MAX_GROUPS];
   double depth[LEGO_GROUPED_MAX_GROUPS], small_cost[LEGO_GROUPED_MAX_GROUPS];
   long total = 0;
   for (int s = 0; s < groups; ++s) {
-    const int g = plan.order[s];
+    const int g = order[s];
     const int m = sizes3[3 * g], n = sizes3[3 * g + 1];
     big[s] = static_cast<long>((m + 255) / 256) * ((n + 255) / 256);
     small[s] = static_cast<long>((m + 127) / 128) * ((n + 127) / 128);
@@ -729,13 +772,39 @@ GroupedPlan grouped_plan(const int* sizes3, int groups)
   return plan;
 }
 
+// The plan is a few hundred list-scheduling steps per candidate split, tens of microseconds of host time in front
+// of a launch of about a hundred: a serving loop calls with the same sizes again and again, so the last few plans
+// are kept, keyed by the sizes themselves.
+GroupedPlan grouped_plan(const int* sizes3, int groups)
+{
+  struct Kept { int groups; int sizes[3 * LEGO_GROUPED_MAX_GROUPS]; GroupedPlan plan; };
+  constexpr int kKept = 8;
+  static Kept kept[kKept];
+  static int next = 0;
+  static std::mutex kept_mutex;
+  const size_t bytes = sizeof(int) * 3 * static_cast<size_t>(groups);
+  {
+    std::lock_guard<std::mutex> hold(kept_mutex);
+    for (int i = 0; i < kKept; ++i)
+      if (kept[i].groups == groups && memcmp(kept[i].sizes, sizes3, bytes) == 0) return kept[i].plan;
+  }
+  const GroupedPlan plan = grouped_plan_uncached(sizes3, groups);
+  std::lock_guard<std::mutex> hold(kept_mutex);
+  Kept& slot = kept[next];
+  next = (next + 1) % kKept;
+  slot.groups = groups;
+  memcpy(slot.sizes, sizes3, bytes);
+  slot.plan = plan;
+  return plan;
+}
+
 // 0: every problem fits the tiled kernels (one launch); 2: the arguments are valid but some problem needs
 // the element-wise kernel (N or K not in whole 16-byte chunks, a base that is not 16-byte aligned);
 // kInvalid otherwise
 int grouped_check(const void* const* a, const void* const* b, void* const* c, const int* sizes3, int groups)
 {
   if (a == nullptr || b == nullptr || c == nullptr || sizes3 == nullptr) return kInvalid;
-  if (groups <= 0 || groups > LEGO_GROUPED_MAX_GROUPS) return kInvalid;
+  if (groups <= 0 || groups > kGroupedMaxProblems) return kInvalid;
   int verdict = 0;
   for (int g = 0; g < groups; ++g) {
     const int m = sizes3[3 * g], n = sizes3[3 * g + 1], k = sizes3[3 * g + 2];
@@ -761,12 +830,41 @@ int grouped_one_by_one(const void* const* a, const void* const* b, void* const* 
 }
 }  // namespace
 
+namespace {
+// More problems than one launch carries (the reference's host function takes any number: its tables live in
+// device memory, grouped_gemm.py:120-162): all problems in order of decreasing depth (stable), cut into runs of
+// LEGO_GROUPED_MAX_GROUPS, one launch per run on the same stream -- so every launch still starts with its longest
+// tiles, and only the last launches hold the shallow problems whose tail rounds are short.
+int grouped_in_runs(const void* const* a, const void* const* b, void* const* c, const int* sizes3, int groups, void* stream)
+{
+  std::vector<int> order(static_cast<size_t>(groups));
+  for (int g = 0; g < groups; ++g) order[static_cast<size_t>(g)] = g;
+  std::stable_sort(order.begin(), order.end(), [sizes3](int p, int q) { return sizes3[3 * p + 2] > sizes3[3 * q + 2]; });
+  const void* ra[LEGO_GROUPED_MAX_GROUPS];
+  const void* rb[LEGO_GROUPED_MAX_GROUPS];
+  void* rc[LEGO_GROUPED_MAX_GROUPS];
+  int rs[3 * LEGO_GROUPED_MAX_GROUPS];
+  for (int first = 0; first < groups; first += LEGO_GROUPED_MAX_GROUPS) {
+    const int count = groups - first < LEGO_GROUPED_MAX_GROUPS ? groups - first : LEGO_GROUPED_MAX_GROUPS;
+    for (int i = 0; i < count; ++i) {
+      const int g = order[static_cast<size_t>(first + i)];
+      ra[i] = a[g]; rb[i] = b[g]; rc[i] = c[g];
+      rs[3 * i] = sizes3[3 * g]; rs[3 * i + 1] = sizes3[3 * g + 1]; rs[3 * i + 2] = sizes3[3 * g + 2];
+    }
+    const int err = lego_hip_grouped_gemm_f16(ra, rb, rc, rs, count, stream);
+    if (err != 0) return err;
+  }
+  return 0;
+}
+}  // namespace
+
 int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* const* c,
                               const int* sizes3, int groups, void* stream)
 {
   const int checked = grouped_check(a, b, c, sizes3, groups);
   if (checked == 2) return grouped_one_by_one(a, b, c, sizes3, groups, stream);
   if (checked != 0) return kInvalid;
+  if (groups > LEGO_GROUPED_MAX_GROUPS) return grouped_in_runs(a, b, c, sizes3, groups, stream);
   // One launch: on 256 x 256 tiles (one workgroup per CU), the last tiles of the launch order split
   // into halves when whole tiles would leave the last round mostly empty, or on 128 x 128 tiles (four
   // times as many workgroups of a quarter of the work, two per CU) when the big ones leave most CUs
@@ -794,7 +892,7 @@ int lego_hip_grouped_gemm_f16_plan(const int* sizes3, int groups, int* plan3)
 int lego_hip_grouped_gemm_f16_split(const void* const* a, const void* const* b, void* const* c,
                                     const int* sizes3, int groups, int split_tiles, void* stream)
 {
-  if (grouped_check(a, b, c, sizes3, groups) != 0) return kInvalid;     // tiled problems only
+  if (groups > LEGO_GROUPED_MAX_GROUPS || grouped_check(a, b, c, sizes3, groups) != 0) return kInvalid;     // one launch of tiled problems only
   if (split_tiles < 0)
     return ok_or(lego_grouped_gemm_f16_t128x128_launch(a, b, c, sizes3, groups, as_stream(stream)));
   return ok_or(lego_grouped_gemm_f16_split_launch(a, b, c, sizes3, groups, split_tiles, as_stream(stream)));
@@ -815,6 +913,28 @@ int lego_hip_copy16_stream(const void* in, void* out, unsigned long long bytes, 
   if (!usable(in) || !usable(out) || bytes == 0 || bytes % 16384 || bytes / 16384 > 0x7fffffffull) return kInvalid;
   hipLaunchKernelGGL(lego_copy16_stream_kernel, dim3(static_cast<unsigned>(bytes / 16384)), dim3(256), 0,
                      as_stream(stream), static_cast<const u32x4*>(in), static_cast<u32x4*>(out));
+  return ok_or(hipGetLastError());
+}
+
+int lego_hip_hbm_probe(const void* in, void* out, unsigned long long bytes, int mode, int vectors_per_lane, void* stream)
+{
+  if (!usable(in) || !usable(out) || in == out) return kInvalid;
+  if (mode < 0 || mode > 2 || (vectors_per_lane != 1 && vectors_per_lane != 4)) return kInvalid;
+  const unsigned long long chunk = 4096ull * vectors_per_lane;
+  if (bytes == 0 || bytes % chunk || bytes / chunk > 0x7fffffffull) return kInvalid;
+  const dim3 grid(static_cast<unsigned>(bytes / chunk)), block(256);
+  const u32x4* src = static_cast<const u32x4*>(in);
+  u32x4* dst = static_cast<u32x4*>(out);
+  hipStream_t s = as_stream(stream);
+  if (vectors_per_lane == 1) {
+    if (mode == 0) hipLaunchKernelGGL(lego_probe_read_kernel<1>, grid, block, 0, s, src, dst);
+    else if (mode == 1) hipLaunchKernelGGL(lego_probe_write_kernel<1>, grid, block, 0, s, dst);
+    else hipLaunchKernelGGL(lego_probe_copy_kernel<1>, grid, block, 0, s, src, dst);
+  } else {
+    if (mode == 0) hipLaunchKernelGGL(lego_probe_read_kernel<4>, grid, block, 0, s, src, dst);
+    else if (mode == 1) hipLaunchKernelGGL(lego_probe_write_kernel<4>, grid, block, 0, s, dst);
+    else hipLaunchKernelGGL(lego_probe_copy_kernel<4>, grid, block, 0, s, src, dst);
+  }
   return ok_or(hipGetLastError());
 }
 

@@ -105,6 +105,106 @@ def xcd_remap(per, wg, xcds=XCDS):
     return OrderBy(Col(per, xcds)).TileBy([per, xcds])[j, x]
 
 
+def lane_and_unit(expr, unit_vars, units, lane_vars, lane_values, stride):
+    """Split an LDS offset ``expr`` (unit indices known at generation time, lane indices at run time) into a lane
+    term and two constants per unit: ``expr(u, lane) == add[u] + (lane_term(lane) ^ xor[u])``.
+
+    The XOR-rotated staging layouts have this shape: a unit moves the lane's offset by whole rows (a multiple of
+    ``stride``: an immediate of the LDS instruction) and flips bits of the chunk index inside a row (one v_xor with
+    a literal), so a lane needs one register and one instruction per access where the printed expression costs
+    four or five.  Returns ``(lane_term, {unit: (add, xor)})`` after checking the identity for every unit and every
+    combination of ``lane_values``; raises if the layout does not split this way."""
+    xor_eval = {"BitXor": lambda a, b: int(a) ^ int(b)}
+    lane_term = expr.subs({v: 0 for v in unit_vars})
+    f_lane = sp.lambdify(lane_vars, lane_term, [xor_eval, "math"])
+    f_full = sp.lambdify(list(unit_vars) + list(lane_vars), expr, [xor_eval, "math"])
+    table = {}
+    for u in units:
+        add = xor = None
+        for lv in lane_values:
+            full, base = int(f_full(*u, *lv)), int(f_lane(*lv))
+            if not 0 <= base < stride:
+                raise ValueError("the lane term leaves the first stride")
+            a, x = full // stride * stride, (full % stride) ^ base
+            if add is None:
+                add, xor = a, x
+            elif (a, x) != (add, xor):
+                raise ValueError(f"offset of unit {u} is not stride*n + (lane ^ constant)")
+        table[tuple(u)] = (add, xor)
+    return lane_term, table
+
+
+LAST_KTILE_RING = 8      # vectors a lane holds between reading them back from the staging block and storing them
+
+
+def last_ktile_schedule(TM, TN, NPH, WN):
+    """Slot schedule of a tile's last k-tile, in which the result leaves under the MFMAs.
+
+    The MFMAs go block row by block row (``i``), within a row k-step by k-step: slot ``i*SPR + ks*TN + j``,
+    ``SPR = TN*NPH``, so the accumulators of block row ``i`` are final when row ``i+1`` starts.  A slot also carries
+      loads   during row 0, every operand fragment the k-tile still needs, in the order of their first use (two
+              per slot at first): after row 0 no wave reads the operand buffers any more, and a barrier there
+              hands all of LDS to the staging of the results;
+      stage   during row ``i+1``, block row ``i`` converted and written to the wave's staging block, one unit =
+              four columns of a lane = (block, q) per ``4/NPH`` of a slot;
+      rb, st  during row ``i+2``, the staged rows of block row ``i`` read back as 16-byte vectors (``rb``) and
+              stored to C two slots later (``st``: the LDS latency passes under two MFMAs).
+    What falls past the last row -- the staging of the last block row, the stores of the last two -- is the
+    ``tail``, in the same order without MFMAs.  Returns ``(slots, tail)``; a slot is a dict with the keys
+    ``mfma`` (i, j, ks), ``loads`` [(ks, f)], ``stage`` [(i, j, q)], ``rb`` [it], ``st`` [it], ``barrier``."""
+    assert 4 % NPH == 0 and WN % 16 == 0
+    SPR, U, IPR = TN * NPH, 4 // NPH, WN // 16
+    G = TM * SPR
+    slots = [dict(mfma=None, loads=[], stage=[], rb=[], st=[], barrier=False) for _ in range(G)]
+    for i in range(TM):
+        for ks in range(NPH):
+            for j in range(TN):
+                slots[i * SPR + ks * TN + j]["mfma"] = (i, j, ks)
+    need = []                      # (ks, f): f < TM a fragment of A's block row f, else of B's block column f - TM
+    for ks in range(1, NPH):
+        need += [(ks, 0)] + [(ks, TM + j) for j in range(TN)]
+    for i in range(1, TM):
+        need += [(ks, i) for ks in range(1, NPH)]
+    doubles = max(0, len(need) - SPR)
+    assert doubles <= SPR
+    at = 0
+    for s_ in range(SPR):
+        for _ in range(2 if s_ < doubles else 1):
+            if at < len(need):
+                slots[s_]["loads"].append(need[at])
+                at += 1
+    slots[SPR - 1]["barrier"] = True
+    late = []                      # (global slot, order, kind, payload) of what falls past the last MFMA
+    def put(g, kind, payload):
+        if g < G:
+            slots[g][kind].append(payload)
+        else:
+            late.append((g, len(late), kind, payload))
+    for r in range(TM):
+        for u, (j, q) in enumerate((j, q) for j in range(TN) for q in range(4)):
+            put((r + 1) * SPR + u // U, "stage", (r, j, q))
+        for m in range(IPR):
+            g = (r + 2) * SPR + m * SPR // IPR
+            put(g, "rb", r * IPR + m)
+            put(g + 2, "st", r * IPR + m)
+    # Past the last MFMA nothing hides a latency, so the order is by dependence: the stores whose vectors are already
+    # on their way, then the read-backs of rows staged earlier (up to RING vectors in flight) with the staging of the
+    # last block row behind them, their stores, and the last block row in batches of RING.
+    ordered = [(kind, payload) for _, _, kind, payload in sorted(late)]
+    in_slots = {it for slot in slots for it in slot["rb"]}
+    tail = [(kind, it) for kind, it in ordered if kind == "st" and it in in_slots]
+    early = [it for kind, it in ordered if kind == "rb" and it // IPR < TM - 1]
+    assert len(early) <= LAST_KTILE_RING
+    tail += [("rb", it) for it in early]
+    tail += [(kind, u) for kind, u in ordered if kind == "stage"]
+    tail += [("st", it) for it in early]
+    fresh = [it for kind, it in ordered if kind == "rb" and it // IPR == TM - 1]
+    for first in range(0, len(fresh), LAST_KTILE_RING):
+        batch = fresh[first:first + LAST_KTILE_RING]
+        tail += [("rb", it) for it in batch] + [("st", it) for it in batch]
+    return slots, tail
+
+
 def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped, dtype):
     """Everything the templates need for one tile shape."""
     # element type, bytes per element, k-depth of one MFMA, result type; the 8-bit types are the
@@ -132,7 +232,11 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
     # the phase after the barrier (the first DMA_LAST) and the phase that follows it (the rest).
     SLOTS, FRAGS, COPIES = TM * TN, TM + TN, A_ITERS + B_ITERS
     assert NPH >= 2 and NPH % 2 == 0, "fragments are double buffered by phase parity"
-    DMA_LAST = min(COPIES, SLOTS // 2 if SLOTS >= 2 * FRAGS else SLOTS)
+    # With two phases per k-tile (8-bit operands) the phase before the barrier is the only one a copy issued in it
+    # would have to land in: all copies go behind the barrier, one per slot, and have the whole next phase
+    # (8192^3 e5m2: 2.75 -> 2.92 PFLOP/s).  With four phases the split 8 + 8 measures best (all 16 behind the barrier,
+    # on top of a fragment load in every other slot, overfill the slots: -4 % on fp16).
+    DMA_LAST = min(COPIES, SLOTS if NPH == 2 else SLOTS // 2 if SLOTS >= 2 * FRAGS else SLOTS)
     assert COPIES - DMA_LAST <= SLOTS
 
     def spread(first, count):
@@ -147,6 +251,7 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
         load_slots[f * SLOTS // FRAGS].append(f)
     dma_last, dma_first = spread(0, DMA_LAST), spread(DMA_LAST, COPIES - DMA_LAST)
     none = [[] for _ in range(SLOTS)]
+    last_slots, last_tail = last_ktile_schedule(TM, TN, NPH, WN)
 
     M, N, K = size("M"), size("N"), size("K")
     npm, npn, per_xcd, group_m = size("num_pid_m"), size("num_pid_n"), size("wg_per_xcd"), size("GM")
@@ -202,6 +307,31 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
              OrderBy(Row(WM, WN // 8)).TileBy([WM, WN // 8]).inv(it * 64 + lane_o)]
 
     pm_e, pn_e = launch_order(npm, npn, group_m, pid)
+
+    # The staging block of the results, as the last k-tile's schedule addresses it (elements of the result type):
+    # a unit (i, j, q) writes four columns of a lane, a read-back `it` fetches 16 bytes of row 4*it + lane/16.
+    stage_e = tidy(4 * Cs_L[i * 32 + l32, j * 8 + q * 2 + lhi], rng)
+    back_e = (tidy(4 * Cs_L[cr, 2 * cp], rng) - 4 * (cr % 2)).subs({cr: c_out[0], cp: c_out[1]})
+    lanes_mfma = [(a_, b_) for a_ in range(32) for b_ in range(2)]
+    stage_lane, stage_ax = lane_and_unit(stage_e, (i, j, q), [(a_, b_, c_) for a_ in range(TM) for b_ in range(TN) for c_ in range(4)],
+                                         (l32, lhi), lanes_mfma, 32 * WN)
+    n_its = WM * WN // 8 // 64
+    back_lane, back_ax = lane_and_unit(back_e, (it,), [(a_,) for a_ in range(n_its)], (lane_o,), [(a_,) for a_ in range(64)], 512)      # a wave instruction moves 64 x 8 elements
+
+    def with_constants(kind, payload):
+        if kind == "stage":
+            return tuple(payload) + stage_ax[tuple(payload)]
+        return (payload,) + back_ax[(payload,)] if kind == "rb" else payload
+    for slot_ in last_slots:
+        slot_["stage"] = [with_constants("stage", u) for u in slot_["stage"]]
+        slot_["rb"] = [with_constants("rb", u) for u in slot_["rb"]]
+    last_tail = [(kind, with_constants(kind, u)) for kind, u in last_tail]
+    # C: the wave's first row and column are uniform, a lane adds its row and 16-byte column, a read-back four rows
+    c_full_e = tidy(C_L[pid_m, pid_n, wm * WM + cr, wn * WN + 8 * cp], rng).subs({cr: c_out[0], cp: c_out[1]})
+    c_wave_e = c_full_e.subs({it: 0, lane_o: 0})
+    c_lane_e = c_full_e.subs({pid_m: 0, pid_n: 0, wm: 0, wn: 0, it: 0})
+    c_it_e = sp.expand(c_full_e.subs(it, 1) - c_full_e.subs(it, 0))
+    assert sp.expand(c_full_e - (c_wave_e + c_lane_e + it * c_it_e)) == 0, "C offsets are not wave + lane + it*step"
 
     # memory->LDS: instruction `it` of wave `wave` fills slots (it*WAVES + wave)*64 + lane; the chunk
     # that lives in a slot is the inverse of the LDS layout
@@ -273,6 +403,7 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
         FMT={"e4m3": 0, "e5m2": 1}.get(dtype, 0), dt=dtype, mfma_dt={"bf16h": "bf16"}.get(dtype, dtype), BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
         WM=WM, WN=WN, TM=TM, TN=TN, A_ITERS=A_ITERS, B_ITERS=B_ITERS, DMA_LAST=DMA_LAST,
         load_slots=load_slots, dma_last=dma_last, dma_first=dma_first, dma_none=none, XCDS=XCDS, MAX_GROUPS=MAX_GROUPS,
+        last_slots=last_slots, last_tail=last_tail, RING=LAST_KTILE_RING,
         pid_layout="OrderBy(Col(max(npm//GM,1),1), Col(min(npm,GM),npn)).TileBy([npm,npn]).inv(pid)",
         MAX_GM=max_group_m,
         xcd_layout=f"OrderBy(Col(nwg/{XCDS}, {XCDS})).TileBy([nwg/{XCDS}, {XCDS}])[Row(nwg/{XCDS}, {XCDS}).inv(wg)]",
@@ -290,6 +421,9 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
         c_out_row=code(c_out[0]), c_out_pair=code(c_out[1]),
         c_stage_load=code(tidy(4 * Cs_L[cr, 2 * cp], rng) - 4 * (cr % 2)),
         c_goff=code(tidy(C_L[pid_m, pid_n, wm * WM + cr, wn * WN + 8 * cp], rng)),
+        c_stage_lane=code(stage_lane), c_back_lane=code(back_lane),
+        c_wave=code(c_wave_e), c_lane=code(c_lane_e), c_it_step=code(c_it_e),
+        c_lane_row=code(c_out[0].subs(it, 0)), c_lane_pair=code(c_out[1].subs(it, 0)), C_ROWS_PER_IT=64 // (WN // 8),
         # the four columns that registers 4q..4q+3 of a lane hold of block (i, j): row and first column within the tile
         c_goff_reg=code(tidy(C_L[pid_m, pid_n, idx("row"), idx("col")], {**rng, idx("row"): (0, bm), idx("col"): (0, bn)})),
         xcd_pid=code(tidy(xcd_remap(per_xcd, wg), {wg: (0, per_xcd * XCDS)})), CUS=CUS,

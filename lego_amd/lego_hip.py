@@ -32,6 +32,7 @@ from pathlib import Path
 from .lego import *  # noqa: F401,F403
 from .lego import GroupBy, TritonRange, product, sp
 from .lego_c import LEGOCCodePrinter
+from sympy.printing.precedence import precedence as _precedence
 
 GFX_ARCH = "gfx950"
 HIPCC_FLAGS = [
@@ -48,18 +49,81 @@ JIT_DIR = _PKG_DIR / "lib" / "jit"
 # expression printer
 # ---------------------------------------------------------------------------
 
-class LEGOHipCodePrinter(LEGOCCodePrinter):
-    """Prints index expressions as HIP/C++ integer arithmetic.
+class HipIntegerRules:
+    """Every printing rule an index expression needs to come out as C++ integer arithmetic, as a mixin
+    that goes IN FRONT of any sympy C printer.
 
-    ``lane_vectors`` maps the axis of a ``TritonRange`` to the name of the per-lane
-    scalar that plays the role of that index vector in the kernel (a lane holds one
-    element of a Triton block, so ``tl.arange(0, BM)[:, None]`` becomes, say, ``row``).
-    Without a mapping the vector prints as ``lane<axis>``.
-    """
+    ``LEGOHipCodePrinter`` carries these rules itself instead of inheriting them from the C printer
+    it sits beside: the reference's ``LEGOCCodePrinter`` (lego/lego_c.py:5-38) overrides ``floor`` and
+    ``Pow`` only, so ``Min``/``Max`` -- which the grouped launch order uses
+    (benchmarks/triton/matmul_sympy.py:57-65) -- would print as the C99 printer's ``fmin``/``fmax``, a
+    ``BitXor`` swizzle as an unknown function call, and ``x - 4*Mod(r, 2)`` as ``x - 4*r % 2``.  With
+    the mixin first in the method resolution order the text is the same over either parent, or over
+    ``sympy.printing.c.C99CodePrinter`` directly."""
 
+    def _print_floor(self, expr):
+        num, den = expr.args[0].as_numer_denom()
+        return f"(({self._print(num)})/({self._print(den)}))"
+
+    @staticmethod
+    def _small_power(expr):
+        return expr.is_Pow and expr.exp.is_Integer and 2 <= int(expr.exp) <= 4
+
+    def _print_Pow(self, expr):
+        if self._small_power(expr):      # i*i, as the reference prints it (benchmarks/cuda/nw/needle_kernel.cu:10)
+            return "*".join([self.parenthesize(expr.base, _precedence(expr))] * int(expr.exp))
+        return super()._print_Pow(expr)
+
+    def _print_Mod(self, expr):
+        # an operand printed as a product needs parentheses that sympy's ranking of Pow above % does not ask for
+        parts = []
+        for arg in expr.args:
+            text = self.parenthesize(arg, _precedence(expr))
+            parts.append(f"({text})" if self._small_power(arg) else text)
+        return " % ".join(parts)
+
+    def _print_Mul(self, expr):
+        # sympy picks the parenthesisation level of a product before it strips the sign, so a negative
+        # product's factors would print at the level of a sum: print the positive product on its own
+        coeff, _ = expr.as_coeff_Mul()
+        if coeff.is_negative:
+            positive = -expr
+            text = self._print(positive)
+            return "-(" + text + ")" if isinstance(positive, sp.Mod) else "-" + text
+        return super()._print_Mul(expr)
+
+    def _integer_select(self, args, op):
+        out = self._print(args[0])
+        for a in args[1:]:
+            b = self._print(a)
+            out = f"(({out}) {op} ({b}) ? ({out}) : ({b}))"
+        return out
+
+    def _print_Min(self, expr):
+        return self._integer_select(expr.args, "<")
+
+    def _print_Max(self, expr):
+        return self._integer_select(expr.args, ">")
+
+    def _print_BitXor(self, expr):      # dispatched by the function's name: any integer-valued Function called BitXor
+        a, b = expr.args
+        return f"(({self._print(a)}) ^ ({self._print(b)}))"
+
+
+    # ``lane_vectors`` maps the axis of a ``TritonRange`` to the name of the per-lane scalar that plays the
+    # role of that index vector in the kernel (a lane holds one element of a Triton block, so
+    # ``tl.arange(0, BM)[:, None]`` becomes, say, ``row``).  Without a mapping the vector prints as ``lane<axis>``.
     def __init__(self, settings=None, lane_vectors=None, **kwargs):
         self.lane_vectors = dict(lane_vectors or {})
-        super().__init__(settings, **kwargs)
+        merged = dict(settings or {})
+        merged.update(kwargs)
+        # The parents disagree on how settings arrive: this package's C printer and the reference's
+        # (lego/lego_c.py:6-7) take them as keywords, sympy's own C printers as one positional dict.
+        try:
+            super().__init__(**merged)
+        except TypeError:
+            super().__init__(merged)
+
 
     def _print_TritonRange(self, expr):
         axis = int(expr.args[1]) if expr.args[1].is_Integer else expr.args[1]
@@ -70,6 +134,11 @@ class LEGOHipCodePrinter(LEGOCCodePrinter):
 
     def _print_Relational(self, expr):
         return f"{self._print(expr.lhs)} {expr.rel_op} {self._print(expr.rhs)}"
+
+
+class LEGOHipCodePrinter(HipIntegerRules, LEGOCCodePrinter):
+    """Prints index expressions as HIP/C++ integer arithmetic: ``HipIntegerRules`` over the C printer of the
+    package it is part of (``LEGOHipCodePrinter(lane_vectors={0: "row", 1: "col"}).doprint(expr)``)."""
 
 
 # ---------------------------------------------------------------------------

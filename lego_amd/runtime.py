@@ -62,6 +62,7 @@ SIGNATURES = {
     "lego_hip_layernorm_bwd_bf16": [_c_void_p] * 9 + [ctypes.c_ulonglong, _c_int, _c_int, _c_void_p],
     "lego_hip_copy16": [_c_void_p, _c_void_p, ctypes.c_ulonglong, _c_void_p],
     "lego_hip_copy16_stream": [_c_void_p, _c_void_p, ctypes.c_ulonglong, _c_void_p],
+    "lego_hip_hbm_probe": [_c_void_p, _c_void_p, ctypes.c_ulonglong, _c_int, _c_int, _c_void_p],
 }
 
 _lib = None

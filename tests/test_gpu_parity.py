@@ -52,10 +52,15 @@ def test_transpose_config1_fp32_4096(ops):
 def test_transpose_config2_fp16_16384_properties(ops):
     """Full size: transposing twice is the identity and the result equals the strided view."""
     print("transpose config 2", flush=True)
-    x = torch.randn(16384, 16384, generator=_gen(1)).half().cuda()
+    xc = torch.randn(16384, 16384, generator=_gen(1)).half()
+    x = xc.cuda()
     y = ops.transpose(x)
     assert torch.equal(y, x.t())
     assert torch.equal(ops.transpose(y), x)
+    # and against the CPU path itself on two strips of the matrix: the oracle's index scatter through both
+    # TileBy([.., ..], [64, 64]) layouts on columns 0..255 (rows 0..255 of the result) and the last 256 columns
+    for cols in (slice(0, 256), slice(16384 - 256, 16384)):
+        assert torch.equal(y[cols].cpu(), ok.transpose(xc[:, cols].contiguous(), 64, 64))
 
 
 def test_transpose_windowed_order_rectangular(ops):
@@ -314,7 +319,11 @@ def test_layernorm_fp32_long_rows_through_the_c_abi(ops, N):
 def test_layernorm_matches_oracle(ops, M, N, wpr):
     print(f"layernorm {M}x{N} wpr={wpr}", flush=True)
     if wpr is not None and N > min(8192 * wpr, 16384):
-        pytest.skip("a row must fit the registers of its team")
+        from lego_amd.runtime import LegoHipError
+        z = torch.zeros(M, N, device="cuda", dtype=torch.half)
+        with pytest.raises(LegoHipError):      # a row must fit the registers of its team
+            ops.layer_norm_fwd(z, z[0].clone(), z[0].clone(), 1e-5, waves_per_row=wpr)
+        return
     g = _gen(3)
     x = (2.0 * torch.randn(M, N, generator=g)).half()
     w = (1 + 0.1 * torch.randn(N, generator=g)).half()
@@ -748,20 +757,35 @@ def test_grouped_gemm_entry_point_with_odd_problems(ops):
         assert torch.equal(c.float(), a.float() @ b.float())
 
 
-def test_grouped_gemm_takes_up_to_64_problems(ops):
-    """The most problems one call takes (the kernels' argument block holds 64), all of different shape, many of a
-    single ragged tile; one more is refused."""
-    from lego_amd.runtime import LegoHipError
-    print("grouped gemm, 64 problems", flush=True)
+@pytest.mark.parametrize("count", [64, 65, 130])
+def test_grouped_gemm_takes_any_number_of_problems(ops, count):
+    """One launch carries 64 problems (the kernels' argument block); a call with more is enqueued as runs of 64 in
+    order of decreasing depth, as the reference's host function takes any group size (grouped_gemm.py:120-162).
+    All problems of different shape, many of a single ragged tile, depths unsorted; results come back in the
+    caller's order."""
+    print(f"grouped gemm, {count} problems", flush=True)
     g = _gen(45)
-    shapes = [(8 * (1 + (5 * i) % 37), 8 * (1 + (7 * i) % 29), 8 * (1 + (3 * i) % 23)) for i in range(64)]
+    shapes = [(8 * (1 + (5 * i) % 37), 8 * (1 + (7 * i) % 29), 8 * (1 + (3 * i) % 23)) for i in range(count)]
     A = [torch.randint(-2, 3, (m, k), generator=g).half() for m, n, k in shapes]
     B = [torch.randint(-2, 3, (k, n), generator=g).half() for m, n, k in shapes]
     got = ops.lego_group_gemm_fn([a.cuda() for a in A], [b.cuda() for b in B])
-    for a, b, c in zip(A, B, got):
+    for (m, n, k), a, b, c in zip(shapes, A, B, got):
+        assert c.shape == (m, n)
         assert torch.equal(c.cpu().float(), a.float() @ b.float())      # small integers: exact
-    with pytest.raises(LegoHipError):
-        ops.lego_group_gemm_fn([a.cuda() for a in A + A[:1]], [b.cuda() for b in B + B[:1]])
+        assert torch.equal(c.cpu(), ok.gemm(a, b))
+
+
+def test_grouped_gemm_of_130_problems_against_the_oracle(ops):
+    """More than two runs' worth of problems with fractional data, each against the CPU oracle to the
+    contract's relative error."""
+    print("grouped gemm, 130 problems, random data", flush=True)
+    g = _gen(46)
+    shapes = [(64 * (1 + i % 5), 8 * (3 + (11 * i) % 40), 64 * (1 + (7 * i) % 9)) for i in range(130)]
+    A = [(torch.randn(m, k, generator=g) / math.sqrt(k)).half() for m, n, k in shapes]
+    B = [(torch.randn(k, n, generator=g) / math.sqrt(k)).half() for m, n, k in shapes]
+    got = ops.lego_group_gemm_fn([a.cuda() for a in A], [b.cuda() for b in B])
+    for a, b, c in zip(A, B, got):
+        assert _rel_err(c.cpu(), ok.gemm(a, b)) <= 1e-2
 
 
 def _grouped_call(entry, A, B, *extra):

@@ -155,3 +155,62 @@ def test_loops_carry_values():
                 def loop(pargs, _, carried):
                     return carried[0]
                 loop()
+
+
+def _launch_order_exprs():
+    npm, npn, gm, pid = sp.symbols("num_pid_m num_pid_n GM pid", integer=True, positive=True)
+    return gemm.launch_order(npm, npn, gm, pid)      # benchmarks/triton/matmul_sympy.py:57-65
+
+
+class _ReferenceShapedCPrinter(sp.printing.c.C99CodePrinter):
+    """What the HIP printer finds beside it when its file is dropped into the reference's package: a C99
+    printer that takes its settings as keywords and overrides ``floor`` only, so ``Min``/``Max`` fall
+    through to ``fmin``/``fmax`` (the behaviour of lego/lego_c.py:5-38, restated here in five lines)."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, kwargs)
+
+    def _print_floor(self, expr):
+        num, den = expr.args[0].as_numer_denom()
+        return f"(({self._print(num)})/({self._print(den)}))"
+
+
+@pytest.mark.parametrize("parent", [sp.printing.c.C99CodePrinter, _ReferenceShapedCPrinter])
+def test_hip_rules_print_integers_over_a_stock_c_printer(parent, tmp_path):
+    """The HIP printer's rules do not lean on the C printer they sit on: over sympy's own C99 printer and over
+    one shaped like the reference's (both print Min/Max as fmin/fmax), the grouped launch order still comes out
+    as integer ternaries, character for character what LEGOHipCodePrinter prints, and its value is the
+    reference's generated pid_m / pid_n (triton_generated/matmul/matmul_NTA_NTB.py:108-109)."""
+    from lego_amd.lego_hip import HipIntegerRules
+    from oracle.kernels import grouped_pid
+
+    pm, pn = _launch_order_exprs()
+    assert "fmin" in parent().doprint(pm) or "fmin" in _ReferenceShapedCPrinter().doprint(pm)      # what is being avoided
+    over = type("HipOver" + parent.__name__, (HipIntegerRules, parent), {})
+    pr = over(allow_unknown_functions=True)
+    text_m, text_n = pr.doprint(pm), pr.doprint(pn)
+    ours = LEGOHipCodePrinter(allow_unknown_functions=True)
+    assert (text_m, text_n) == (ours.doprint(pm), ours.doprint(pn))
+    for text in (text_m, text_n):
+        assert "fmin" not in text and "fmax" not in text and "?" in text
+    a, b = sp.symbols("a b", integer=True, positive=True)
+    assert pr.doprint(BitXor(a, 4 * b)) == "((a) ^ (4*b))"
+    assert pr.doprint(a - 4 * sp.Mod(b, 2)) == "a - 4*(b % 2)"
+    assert pr.doprint(sp.Mod(a, b ** 2)) == "a % (b*b)"
+
+    # the printed text is C: compile it with the host compiler and run it over whole launch grids
+    cases = ((32, 32, 8), (16, 8, 8), (8, 16, 4), (4, 4, 8), (6, 5, 3))
+    src = tmp_path / "order.c"
+    src.write_text(
+        "#include <stdio.h>\n"
+        f"static int pm(int pid, int num_pid_m, int num_pid_n, int GM) {{ return {text_m}; }}\n"
+        f"static int pn(int pid, int num_pid_m, int num_pid_n, int GM) {{ return {text_n}; }}\n"
+        "int main(void) {\n"
+        + "".join(f"  for (int pid = 0; pid < {npm * npn}; ++pid) printf(\"%d %d\\n\", pm(pid, {npm}, {npn}, {gm}), pn(pid, {npm}, {npn}, {gm}));\n"
+                  for npm, npn, gm in cases)
+        + "  return 0;\n}\n")
+    exe = tmp_path / "order"
+    subprocess.run(["gcc", "-O1", "-Wall", "-Werror", str(src), "-o", str(exe)], check=True, capture_output=True)
+    got = [tuple(int(v) for v in line.split()) for line in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines()]
+    want = [tuple(int(v) for v in grouped_pid(pid, npm, npn, gm)) for npm, npn, gm in cases for pid in range(npm * npn)]
+    assert got == want
