@@ -4,9 +4,14 @@
  * Conventions for every entry point
  *   - returns 0 on success, otherwise a hipError_t value (1 = hipErrorInvalidValue for a
  *     null pointer, a misaligned base, or a shape the generated kernels do not cover);
- *   - all tensor pointers are BORROWED DEVICE pointers, 16-byte aligned, row-major and
- *     contiguous; nothing is allocated, freed or synchronised: the kernel is enqueued on
- *     `stream` (a hipStream_t; NULL = the default stream) and the call returns;
+ *   - all tensor pointers are BORROWED DEVICE pointers, row-major and contiguous, aligned to
+ *     their element at least (the reference's kernels take any pointer).  16-byte aligned bases
+ *     -- what every allocator hands out -- take the fastest kernels; a base at another element (a
+ *     sliced view) takes the kernels for rows and shapes of any length, which place their
+ *     16-byte accesses where the result has its 16-byte boundaries.  Workspaces and the tuning
+ *     entry points (*_wpr, *_split) ask for 16 bytes.  Nothing is allocated, freed or
+ *     synchronised: the kernel is enqueued on `stream` (a hipStream_t; NULL = the default
+ *     stream) and the call returns;
  *   - re-entrant: safe from several host threads on distinct streams.  Two entry points keep state between
  *     calls, both described where they are declared: lego_hip_lud_f32 (a side stream per caller's stream) and
  *     lego_hip_layernorm_bwd_f16_noalloc (a built-in scratch array per device).
@@ -66,8 +71,9 @@ int lego_hip_layernorm_fwd_bf16(const void* x, void* y, const void* w, const voi
  * allocates its buffers with torch as well): ask for its size first, any 16-byte aligned
  * device buffer of at least that many bytes will do; its contents need no initialisation.
  * Any N up to 32768 (the reference's fp16 limit); rows above 16384 elements are read twice (dx by
- * rows, then dw/db by columns).  Rows of a length that is not a multiple of 8 are split at their 16-byte
- * boundaries, which fall on the same columns in dy, x and dx (16-byte aligned buffers of one shape). */
+ * rows, then dw/db by columns).  Rows of a length that is not a multiple of 8, and tensors at a base that is
+ * not 16-byte aligned, are split where the rows of dx have their 16-byte boundaries (the same columns in dy and x
+ * when all three are 16-byte aligned buffers of one shape).  The workspace size covers either case. */
 int lego_hip_layernorm_bwd_workspace_bytes(int M, int N, unsigned long long* bytes);
 int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, const float* mean,
                                const float* rstd, void* dx, void* dw, void* db, void* workspace,
@@ -81,7 +87,9 @@ int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, con
  * hipErrorInvalidValue).  The device that owns `stream` must be the current device of the calling
  * thread.  Calls on one device share the array: two calls that overlap in time on one device (on
  * different streams) race on it and must be ordered by the caller.  The call itself allocates and
- * frees nothing and does not synchronise. */
+ * frees nothing and does not synchronise.  The first call on a device looks up the array's device address
+ * (hipGetSymbolAddress, which may load the code object that holds the array): make that call outside any
+ * stream capture; the calls after it only enqueue kernels and can be captured. */
 int lego_hip_layernorm_bwd_f16_noalloc(const void* dy, const void* x, const void* w, const float* mean,
                                        const float* rstd, void* dx, void* dw, void* db, int M, int N, void* stream);
 

@@ -90,6 +90,7 @@ def collect():
                 # smaller matrices have too few of these macro tiles: the 64x64 ones of the any-shape kernels are ahead up
                 # to about 32 Mi elements (fp16 2056^2 3.2 against 2.3 TB/s, 4104^2 4.2 / 3.8; 6152^2 3.7 / 4.0)
                 meta["min_elements"] = 32 << 20
+            meta["any_element"] = bool(cfg.get("ragged"))
             if cfg.get("ragged"):     # any shape with at least one whole vector per row of both matrices
                 meta["row_multiple"] = meta["col_multiple"] = 1
                 meta["min_side"] = vec
@@ -151,6 +152,14 @@ def collect():
                 fits += f" && 1ull * rows * cols >= {m['min_elements']}ull"
             h.append(f"  if (rows % {m['row_multiple']} == 0 && cols % {m['col_multiple']} == 0{fits}) "
                      f"return {m['kernel']}_launch(in, out, rows, cols, stream);")
+        h += [f"  return lego_transpose_any_launch(in, out, rows, cols, {4 if dtype == 'f32' else 2}, stream);", "}",
+              "// matrices whose base is only element aligned (a sliced view): the tilings whose vectors sit at any element",
+              f"inline hipError_t lego_transpose_{dtype}_dispatch_any_base(const void* in, void* out, int rows, int cols, "
+              "hipStream_t stream) {"]
+        for m in metas:
+            if m["any_element"]:
+                h.append(f"  if (rows >= {m['min_side']} && cols >= {m['min_side']} && 1ull * rows * cols >= {m['min_elements']}ull) "
+                         f"return {m['kernel']}_launch(in, out, rows, cols, stream);")
         h += [f"  return lego_transpose_any_launch(in, out, rows, cols, {4 if dtype == 'f32' else 2}, stream);", "}", ""]
     for dtype, vec, w in ROWWISE:
         tag = dtype if vec else dtype + "s"
@@ -181,11 +190,11 @@ def collect():
     h += ["unsigned lego_layernorm_bwd_groups(int M, int N);", "unsigned lego_layernorm_bwd_f32_groups(int M, int N);",
           "unsigned lego_layernorm_bwd_bf16_groups(int M, int N);",
           "hipError_t lego_layernorm_bwd_f32_launch(const void*, const void*, const void*, const float*, const float*, "
-          "void*, void*, void*, float*, int, int, hipStream_t);",
+          "void*, void*, void*, float*, int, int, int, hipStream_t);",
           "hipError_t lego_layernorm_bwd_bf16_launch(const void*, const void*, const void*, const float*, const float*, "
-          "void*, void*, void*, float*, int, int, hipStream_t);",
+          "void*, void*, void*, float*, int, int, int, hipStream_t);",
           "hipError_t lego_layernorm_bwd_f16_launch(const void*, const void*, const void*, const float*, const float*, "
-          "void*, void*, void*, float*, int, int, hipStream_t);",
+          "void*, void*, void*, float*, int, int, int, hipStream_t);",
           f"#define LEGO_LAYERNORM_BWD_MAX_N {mlb['MAX_N']}", ""]
     h += [f"hipError_t lego_gemm_{d}_{v}{t}_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);"
           for d in GEMM_DTYPES for v in ("nn", "nt", "tn", "tt")

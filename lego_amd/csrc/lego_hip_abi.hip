@@ -21,6 +21,9 @@ namespace {
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline bool usable(const void* p) { return p != nullptr && aligned16(p); }
+// a tensor base that only has its elements' alignment (a sliced view): the kernels for rows and shapes of any
+// length take those, with 16-byte accesses wherever their result has its 16-byte boundaries
+inline bool element_aligned(const void* p, unsigned bytes) { return p != nullptr && (reinterpret_cast<uintptr_t>(p) & (bytes - 1u)) == 0; }
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 inline int ok_or(hipError_t e) { return static_cast<int>(e); }
 constexpr int kInvalid = static_cast<int>(hipErrorInvalidValue);
@@ -184,15 +187,19 @@ int lego_hip_abi_version(void) { return 1; }
 
 int lego_hip_transpose_f32(const void* in, void* out, int rows, int cols, void* stream)
 {
-  if (!usable(in) || !usable(out) || in == out) return kInvalid;
+  if (!element_aligned(in, 4) || !element_aligned(out, 4) || in == out) return kInvalid;
   if (rows <= 0 || cols <= 0) return kInvalid;
+  if (!aligned16(in) || !aligned16(out))      // a base at any element: the kernels whose vectors sit at any element
+    return ok_or(lego_transpose_f32_dispatch_any_base(in, out, rows, cols, as_stream(stream)));
   return ok_or(lego_transpose_f32_dispatch(in, out, rows, cols, as_stream(stream)));
 }
 
 int lego_hip_transpose_f16(const void* in, void* out, int rows, int cols, void* stream)
 {
-  if (!usable(in) || !usable(out) || in == out) return kInvalid;
+  if (!element_aligned(in, 2) || !element_aligned(out, 2) || in == out) return kInvalid;
   if (rows <= 0 || cols <= 0) return kInvalid;
+  if (!aligned16(in) || !aligned16(out))
+    return ok_or(lego_transpose_f16_dispatch_any_base(in, out, rows, cols, as_stream(stream)));
   return ok_or(lego_transpose_f16_dispatch(in, out, rows, cols, as_stream(stream)));
 }
 
@@ -214,10 +221,10 @@ int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per
 
 int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream)
 {
-  if (!usable(x) || !usable(y) || M <= 0 || N <= 0) return kInvalid;
+  if (!element_aligned(x, 2) || !element_aligned(y, 2) || M <= 0 || N <= 0) return kInvalid;
   if (N > LEGO_ROWWISE_MAX_N) return ok_or(lego_softmax_long_f16_launch(x, y, M, N, as_stream(stream)));   // two passes
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
-  if (N % 8)   // ragged rows
+  if (N % 8 || !aligned16(x) || !aligned16(y))   // rows of any length, or at any element
     return ok_or((N <= 128 ? lego_softmax_f16s_l16_launch : N <= 256 ? lego_softmax_f16s_l32_launch
                   : lego_rowwise_f16_wpr(M, N) == 8 ? lego_softmax_f16s_w8_launch
                   : long_row ? lego_softmax_f16s_w16_launch : lego_rowwise_default_wpr(N) == 1 ? lego_softmax_f16s_w1_launch
@@ -228,10 +235,10 @@ int lego_hip_softmax_f16(const void* x, void* y, int M, int N, void* stream)
 
 int lego_hip_softmax_f32(const void* x, void* y, int M, int N, void* stream)
 {
-  if (!usable(x) || !usable(y) || M <= 0 || N <= 0) return kInvalid;
+  if (!element_aligned(x, 4) || !element_aligned(y, 4) || M <= 0 || N <= 0) return kInvalid;
   if (N > LEGO_ROWWISE_MAX_N) return ok_or(lego_softmax_long_f32_launch(x, y, M, N, as_stream(stream)));   // two passes
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
-  if (N % 4)   // ragged rows
+  if (N % 4 || !aligned16(x) || !aligned16(y))   // rows of any length, or at any element
     return ok_or((N <= 64 ? lego_softmax_f32s_l16_launch : N <= 128 ? lego_softmax_f32s_l32_launch
                   : lego_rowwise_f16_wpr(M, 2 * N) == 8 ? lego_softmax_f32s_w8_launch
                   : long_row ? lego_softmax_f32s_w16_launch : N <= 1024 ? lego_softmax_f32s_w1_launch
@@ -267,10 +274,11 @@ int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const 
 int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void* b,
                                float* mean, float* rstd, int M, int N, float eps, void* stream)
 {
-  if (!usable(x) || !usable(y) || !usable(w) || !usable(b) || mean == nullptr || rstd == nullptr) return kInvalid;
+  if (!element_aligned(x, 2) || !element_aligned(y, 2) || !element_aligned(w, 2) || !element_aligned(b, 2)) return kInvalid;
+  if (!element_aligned(mean, 4) || !element_aligned(rstd, 4)) return kInvalid;
   if (M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
-  if (N % 8)   // ragged rows
+  if (N % 8 || !aligned16(x) || !aligned16(y) || !aligned16(w) || !aligned16(b))   // rows of any length, or at any element
     return ok_or((N <= 128 ? lego_layernorm_fwd_f16s_l16_launch : N <= 256 ? lego_layernorm_fwd_f16s_l32_launch
                   : lego_rowwise_f16_wpr(M, N) == 8 ? lego_layernorm_fwd_f16s_w8_launch
                   : long_row ? lego_layernorm_fwd_f16s_w16_launch : lego_rowwise_default_wpr(N) == 1 ? lego_layernorm_fwd_f16s_w1_launch
@@ -282,10 +290,11 @@ int lego_hip_layernorm_fwd_f16(const void* x, void* y, const void* w, const void
 int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void* b,
                                float* mean, float* rstd, int M, int N, float eps, void* stream)
 {
-  if (!usable(x) || !usable(y) || !usable(w) || !usable(b) || mean == nullptr || rstd == nullptr) return kInvalid;
+  if (!element_aligned(x, 4) || !element_aligned(y, 4) || !element_aligned(w, 4) || !element_aligned(b, 4)) return kInvalid;
+  if (!element_aligned(mean, 4) || !element_aligned(rstd, 4)) return kInvalid;
   if (M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
   const bool long_row = N > LEGO_ROWWISE_MAX_N_SMALL_TEAMS;
-  if (N % 4)   // ragged rows
+  if (N % 4 || !aligned16(x) || !aligned16(y) || !aligned16(w) || !aligned16(b))   // rows of any length, or at any element
     return ok_or((N <= 64 ? lego_layernorm_fwd_f32s_l16_launch : N <= 128 ? lego_layernorm_fwd_f32s_l32_launch
                   : lego_rowwise_f16_wpr(M, 2 * N) == 8 ? lego_layernorm_fwd_f32s_w8_launch
                   : long_row ? lego_layernorm_fwd_f32s_w16_launch : N <= 1024 ? lego_layernorm_fwd_f32s_w1_launch
@@ -303,10 +312,10 @@ int lego_hip_layernorm_fwd_f32(const void* x, void* y, const void* w, const void
 
 int lego_hip_softmax_bf16(const void* x, void* y, int M, int N, void* stream)
 {
-  if (!usable(x) || !usable(y) || M <= 0 || N <= 0) return kInvalid;
+  if (!element_aligned(x, 2) || !element_aligned(y, 2) || M <= 0 || N <= 0) return kInvalid;
   if (N > LEGO_ROWWISE_MAX_N) return ok_or(lego_softmax_long_bf16_launch(x, y, M, N, as_stream(stream)));   // two passes
   const int wpr = lego_rowwise_default_wpr(N);
-  if (N % 8)   // ragged rows
+  if (N % 8 || !aligned16(x) || !aligned16(y))   // rows of any length, or at any element
     return ok_or((N <= 128 ? lego_softmax_bf16s_l16_launch : N <= 256 ? lego_softmax_bf16s_l32_launch
                   : lego_rowwise_f16_wpr(M, N) == 8 ? lego_softmax_bf16s_w8_launch
                   : wpr == 16 ? lego_softmax_bf16s_w16_launch : wpr == 1 ? lego_softmax_bf16s_w1_launch
@@ -320,10 +329,11 @@ int lego_hip_softmax_bf16(const void* x, void* y, int M, int N, void* stream)
 int lego_hip_layernorm_fwd_bf16(const void* x, void* y, const void* w, const void* b,
                                 float* mean, float* rstd, int M, int N, float eps, void* stream)
 {
-  if (!usable(x) || !usable(y) || !usable(w) || !usable(b) || mean == nullptr || rstd == nullptr) return kInvalid;
+  if (!element_aligned(x, 2) || !element_aligned(y, 2) || !element_aligned(w, 2) || !element_aligned(b, 2)) return kInvalid;
+  if (!element_aligned(mean, 4) || !element_aligned(rstd, 4)) return kInvalid;
   if (M <= 0 || N <= 0 || N > LEGO_ROWWISE_MAX_N || !(eps >= 0.0f)) return kInvalid;
   const int wpr = lego_rowwise_default_wpr(N);
-  if (N % 8)   // ragged rows
+  if (N % 8 || !aligned16(x) || !aligned16(y) || !aligned16(w) || !aligned16(b))   // rows of any length, or at any element
     return ok_or((N <= 128 ? lego_layernorm_fwd_bf16s_l16_launch : N <= 256 ? lego_layernorm_fwd_bf16s_l32_launch
                   : lego_rowwise_f16_wpr(M, N) == 8 ? lego_layernorm_fwd_bf16s_w8_launch
                   : wpr == 16 ? lego_layernorm_fwd_bf16s_w16_launch : wpr == 1 ? lego_layernorm_fwd_bf16s_w1_launch
@@ -353,10 +363,12 @@ int lego_hip_layernorm_bwd_f16(const void* dy, const void* x, const void* w, con
 {
   unsigned long long need = 0;
   if (lego_hip_layernorm_bwd_workspace_bytes(M, N, &need) != 0) return kInvalid;
-  if (!usable(dy) || !usable(x) || !usable(w) || !usable(dx) || !usable(dw) || !usable(db) || !usable(workspace))
+  if (!element_aligned(dy, 2) || !element_aligned(x, 2) || !element_aligned(w, 2) || !element_aligned(dx, 2) ||
+      !element_aligned(dw, 2) || !element_aligned(db, 2) || !usable(workspace))
     return kInvalid;
-  if (mean == nullptr || rstd == nullptr || workspace_bytes < need) return kInvalid;
-  return ok_or(lego_layernorm_bwd_f16_launch(dy, x, w, mean, rstd, dx, dw, db, static_cast<float*>(workspace), M, N,
+  if (!element_aligned(mean, 4) || !element_aligned(rstd, 4) || workspace_bytes < need) return kInvalid;
+  const int any_base = !(aligned16(dy) && aligned16(x) && aligned16(w) && aligned16(dx));
+  return ok_or(lego_layernorm_bwd_f16_launch(dy, x, w, mean, rstd, dx, dw, db, static_cast<float*>(workspace), M, N, any_base,
                                              as_stream(stream)));
 }
 
@@ -366,14 +378,17 @@ int lego_hip_layernorm_bwd_f16_noalloc(const void* dy, const void* x, const void
   unsigned long long need = 0;
   if (lego_hip_layernorm_bwd_workspace_bytes(M, N, &need) != 0) return kInvalid;
   if (need > kScratchBytes) return kInvalid;     // partial rows beyond the built-in scratch
-  if (!usable(dy) || !usable(x) || !usable(w) || !usable(dx) || !usable(dw) || !usable(db)) return kInvalid;
-  if (mean == nullptr || rstd == nullptr) return kInvalid;
+  if (!element_aligned(dy, 2) || !element_aligned(x, 2) || !element_aligned(w, 2) || !element_aligned(dx, 2) ||
+      !element_aligned(dw, 2) || !element_aligned(db, 2))
+    return kInvalid;
+  if (!element_aligned(mean, 4) || !element_aligned(rstd, 4)) return kInvalid;
+  const int any_base = !(aligned16(dy) && aligned16(x) && aligned16(w) && aligned16(dx));
   float* partials = nullptr;
   const hipError_t err = scratch_address(&partials);
   if (err != hipSuccess) return ok_or(err);
   // every partial row that the reduction reads is written by the first stage of the same call, so
   // what an earlier call left in the array needs no clearing
-  return ok_or(lego_layernorm_bwd_f16_launch(dy, x, w, mean, rstd, dx, dw, db, partials, M, N, as_stream(stream)));
+  return ok_or(lego_layernorm_bwd_f16_launch(dy, x, w, mean, rstd, dx, dw, db, partials, M, N, any_base, as_stream(stream)));
 }
 
 int lego_hip_layernorm_bwd_f32_workspace_bytes(int M, int N, unsigned long long* bytes)
@@ -390,10 +405,12 @@ int lego_hip_layernorm_bwd_f32(const void* dy, const void* x, const void* w, con
 {
   unsigned long long need = 0;
   if (lego_hip_layernorm_bwd_f32_workspace_bytes(M, N, &need) != 0) return kInvalid;
-  if (!usable(dy) || !usable(x) || !usable(w) || !usable(dx) || !usable(dw) || !usable(db) || !usable(workspace))
+  if (!element_aligned(dy, 4) || !element_aligned(x, 4) || !element_aligned(w, 4) || !element_aligned(dx, 4) ||
+      !element_aligned(dw, 4) || !element_aligned(db, 4) || !usable(workspace))
     return kInvalid;
-  if (mean == nullptr || rstd == nullptr || workspace_bytes < need) return kInvalid;
-  return ok_or(lego_layernorm_bwd_f32_launch(dy, x, w, mean, rstd, dx, dw, db, static_cast<float*>(workspace), M, N,
+  if (!element_aligned(mean, 4) || !element_aligned(rstd, 4) || workspace_bytes < need) return kInvalid;
+  const int any_base = !(aligned16(dy) && aligned16(x) && aligned16(w) && aligned16(dx));
+  return ok_or(lego_layernorm_bwd_f32_launch(dy, x, w, mean, rstd, dx, dw, db, static_cast<float*>(workspace), M, N, any_base,
                                              as_stream(stream)));
 }
 
@@ -411,10 +428,12 @@ int lego_hip_layernorm_bwd_bf16(const void* dy, const void* x, const void* w, co
 {
   unsigned long long need = 0;
   if (lego_hip_layernorm_bwd_bf16_workspace_bytes(M, N, &need) != 0) return kInvalid;
-  if (!usable(dy) || !usable(x) || !usable(w) || !usable(dx) || !usable(dw) || !usable(db) || !usable(workspace))
+  if (!element_aligned(dy, 2) || !element_aligned(x, 2) || !element_aligned(w, 2) || !element_aligned(dx, 2) ||
+      !element_aligned(dw, 2) || !element_aligned(db, 2) || !usable(workspace))
     return kInvalid;
-  if (mean == nullptr || rstd == nullptr || workspace_bytes < need) return kInvalid;
-  return ok_or(lego_layernorm_bwd_bf16_launch(dy, x, w, mean, rstd, dx, dw, db, static_cast<float*>(workspace), M, N,
+  if (!element_aligned(mean, 4) || !element_aligned(rstd, 4) || workspace_bytes < need) return kInvalid;
+  const int any_base = !(aligned16(dy) && aligned16(x) && aligned16(w) && aligned16(dx));
+  return ok_or(lego_layernorm_bwd_bf16_launch(dy, x, w, mean, rstd, dx, dw, db, static_cast<float*>(workspace), M, N, any_base,
                                               as_stream(stream)));
 }
 

@@ -36,7 +36,12 @@ def test_argument_validation_needs_no_gpu():
     assert lib.lego_hip_transpose_f32(None, None, 64, 64, None) == 1
     assert lib.lego_hip_transpose_f16(ctypes.c_void_p(16), ctypes.c_void_p(4096), 0, 64, None) == 1
     assert lib.lego_hip_transpose_f16(ctypes.c_void_p(4096), ctypes.c_void_p(4096), 64, 64, None) == 1   # in place
-    assert lib.lego_hip_transpose_f16(ctypes.c_void_p(8), ctypes.c_void_p(4096), 64, 64, None) == 1
+    assert lib.lego_hip_transpose_f16(ctypes.c_void_p(4097), ctypes.c_void_p(4096), 64, 64, None) == 1   # not even element aligned
+    assert lib.lego_hip_transpose_f32(ctypes.c_void_p(4098), ctypes.c_void_p(8192), 64, 64, None) == 1
+    assert lib.lego_hip_softmax_f16(ctypes.c_void_p(4097), ctypes.c_void_p(8192), 4, 64, None) == 1
+    assert lib.lego_hip_layernorm_fwd_f32(ctypes.c_void_p(4096), ctypes.c_void_p(8194), ctypes.c_void_p(64), ctypes.c_void_p(128),
+                                          ctypes.c_void_p(256), ctypes.c_void_p(512), 4, 64, ctypes.c_float(1e-5), None) == 1
+    assert lib.lego_hip_softmax_f16_wpr(ctypes.c_void_p(4098), ctypes.c_void_p(8192), 4, 64, 1, None) == 1   # the tuning entry points keep 16 bytes
     assert lib.lego_hip_softmax_f16(ctypes.c_void_p(16), ctypes.c_void_p(4096), 4, 0, None) == 1
     assert lib.lego_hip_softmax_f16_wpr(ctypes.c_void_p(16), ctypes.c_void_p(4096), 4, 12, 4, None) == 1
     assert lib.lego_hip_softmax_f32(ctypes.c_void_p(16), ctypes.c_void_p(4096), 0, 64, None) == 1
