@@ -64,9 +64,10 @@ def main():
     ap.add_argument("--sustain", type=float, default=0.0, metavar="SECONDS",
                     help="after timing the 8192^3 GEMM, keep launching it back to back for this long (for sampling "
                          "socket power and clocks with amd-smi from another process) and report the sustained rate")
-    ap.add_argument("--only", default="", help="comma list of configs to time (c1,c2,c3,c4,c5,extra,apps); "
+    ap.add_argument("--only", default="", help="comma list of configs to time (c1,c2,c3,c4,c5,extra,apps,energy); "
                     "c2 is always timed; 'extra' adds LayerNorm backward and the other GEMM layouts and element "
-                    "types, 'apps' the stencil, Needleman-Wunsch and LUD programs")
+                    "types, 'apps' the stencil, Needleman-Wunsch and LUD programs, 'energy' (with c4) the sustained "
+                    "comparison of GEMM variants and MFMA-only streams for power sampling")
     ns = ap.parse_args()
     if ns.gpus != 1:
         print("bench.py: this build measures one MI355X; every configuration of the hot path is a "
@@ -86,7 +87,7 @@ def main():
     def want(name):
         return not only or name in only
 
-    def timed(fn, steps=K, warmup=W):
+    def timed(fn, steps=K, warmup=W, settle_ms=None):
         """Average milliseconds per call over exactly ``steps`` calls timed with events on the launch
         stream.  Untimed before them: ``warmup`` calls, then as many more as fill SETTLE_MS of device
         time, queued back to back with the timed ones -- after an idle gap the part needs about 20 ms
@@ -100,7 +101,8 @@ def main():
         stop.record()
         torch.cuda.synchronize()
         per_call = start.elapsed_time(stop) / max(1, warmup)
-        for _ in range(min(5000, int(ns.settle_ms / max(per_call, 1e-3)) + 1) if ns.settle_ms > 0 else 0):
+        settle = ns.settle_ms if settle_ms is None else settle_ms
+        for _ in range(min(5000, int(settle / max(per_call, 1e-3)) + 1) if settle > 0 else 0):
             fn()
         start.record()
         for _ in range(steps):
@@ -367,7 +369,28 @@ def main():
             runtime.call("lego_hip_gemm_f16", p(a4), p(b4s), p(c4), n4, n4, n4, stream)
         ms_s = timed(gms, steps=max(5, K // 5), warmup=max(2, W // 5))
         lib_ms_s = timed(lambda: torch.matmul(a4, b4s, out=c4), steps=max(5, K // 5), warmup=max(2, W // 5))
+        # What the matrix cores sustain on operands of this distribution when a kernel issues nothing but MFMAs (one wave
+        # per SIMD, 256 accumulator registers, fragments loaded once): the rate that the part's power management
+        # leaves to an fp16 GEMM whose data movement costs nothing.
+        probe_wgs, probe_iters = 256, 2048
+        probe_ops = (torch.randn(probe_wgs * 32768, generator=g4) / math.sqrt(n4)).half().to(dev)
+        probe_sink = torch.empty(probe_wgs * 512, device=dev)
+        # flop per launch: one MFMA per accumulator block and round, 32 k-values deep for 16x16x32, 16 for 32x32x16
+        probe_flop = {shape: probe_wgs * probe_iters * (4194304.0 if shape in (1, 3) else 2097152.0) for shape in range(5)}
+
+        def mfma_only(shape):
+            return lambda: runtime.call("lego_hip_mfma_probe", p(probe_ops), p(probe_sink), shape, probe_iters, probe_wgs, stream)
+        ms_probe = timed(mfma_only(1), steps=max(5, K // 5), warmup=max(2, W // 5))
+        ms_probe32 = timed(mfma_only(0), steps=max(5, K // 5), warmup=max(2, W // 5))
+        mfma_achievable = probe_flop[1] / ms_probe / 1e9
+        kernels["mfma_ceiling_f16"] = dict(
+            ms=ms_probe, tflops=mfma_achievable, frac_mfma=mfma_achievable / MFMA_F16_PEAK_TFLOPS,
+            tflops_32x32x16=probe_flop[0] / ms_probe32 / 1e9,
+            note="v_mfma_f32_16x16x32_f16 only (the GEMM kernels' instruction), 256 workgroups of four waves, operands "
+                 "N(0,1)/sqrt(8192) held in registers: what the part sustains at its power and current limits with the "
+                 "pipe full; tflops_32x32x16 = the same with v_mfma_f32_32x32x16_f16")
         kernels["c4_gemm_f16_8192"] = dict(ms=ms, tflops=fl4 / ms / 1e9, frac_mfma=fl4 / ms / 1e9 / MFMA_F16_PEAK_TFLOPS,
+                                           achievable_tflops=mfma_achievable, frac_of_achievable=fl4 / ms / 1e9 / mfma_achievable,
                                            flop=fl4, rel_err_vs_fp32=rel,
                                            vendor_library_tflops=fl4 / lib_ms / 1e9,
                                            b_address=f"a + {b4.data_ptr() - a4.data_ptr()} bytes",
@@ -375,7 +398,7 @@ def main():
                                            vendor_library_tflops_b_moved_128_bytes=fl4 / lib_ms_s / 1e9,
                                            note="vendor_library = torch.matmul (hipBLASLt) on the same buffers")
         del b4s, b4s_buf
-        if ns.sustain > 0:
+        if ns.sustain > 0 and "energy" not in only:
             for name, fn in (("sustained", gm), ("vendor_library_sustained", lambda: torch.matmul(a4, b4, out=c4))):
                 per = []
                 t_end = time.perf_counter() + ns.sustain
@@ -384,6 +407,41 @@ def main():
                 kernels["c4_gemm_f16_8192"][name + "_tflops"] = fl4 / (sum(per) / len(per)) / 1e9
                 kernels["c4_gemm_f16_8192"][name + "_seconds"] = ns.sustain
                 time.sleep(1.0)      # an idle second between the two, visible in the power samples
+        if "energy" in only:
+            # Energy-per-flop comparison: every variant back to back for --sustain seconds (default 3) with an idle second
+            # between, wall-clock times recorded so that socket power and clocks sampled by another process (amd-smi in a
+            # loop) can be laid beside them; counters for the same kernels come from a rocprofv3 --pmc run of this leg.
+            seconds = ns.sustain if ns.sustain > 0 else 3.0
+            c4w = torch.empty_like(c4)
+            def variant(v, out):
+                return lambda: runtime.call("lego_hip_gemm_f16_variant", p(a4), p(b4), p(out), n4, n4, n4, v, stream)
+            for v in (1, 2):
+                variant(v, c4w)()
+                torch.cuda.synchronize()
+                assert ((c4w[:512].float() - ref).norm() / ref.norm()).item() <= 1e-2
+            phases = [("gemm 8192^3: 4 waves of 128x128, one per SIMD, 16x16x32 MFMA (built)", fl4, variant(0, c4)),
+                      ("gemm 8192^3: 4 waves of 128x128, one per SIMD, 32x32x16 MFMA", fl4, variant(1, c4w)),
+                      ("gemm 8192^3: 8 waves of 128x64, two per SIMD, 32x32x16 MFMA", fl4, variant(2, c4w)),
+                      ("gemm 8192^3: vendor library (torch.matmul)", fl4, lambda: torch.matmul(a4, b4, out=c4)),
+                      ("MFMA only: 32x32x16 f16, one wave per SIMD", probe_flop[0], mfma_only(0)),
+                      ("MFMA only: 16x16x32 f16, one wave per SIMD", probe_flop[1], mfma_only(1)),
+                      ("MFMA only: 32x32x16 f16, two waves per SIMD", probe_flop[4], mfma_only(4)),
+                      ("MFMA only: 16x16x32 f16, two waves per SIMD", probe_flop[3], mfma_only(3)),
+                      ("MFMA only: 32x32x16 bf16 (the same bits), one wave per SIMD", probe_flop[2], mfma_only(2))]
+            table = []
+            for label, flop, fn in phases:
+                per = []
+                t_begin = time.time()
+                t_end = time.perf_counter() + seconds
+                while time.perf_counter() < t_end:
+                    per.append(timed(fn, steps=20, warmup=1, settle_ms=0.0))
+                steady = per[len(per) // 3:]
+                table.append(dict(variant=label, tflops=flop / (sum(steady) / len(steady)) / 1e9, wall_clock_begin=t_begin,
+                                  wall_clock_end=time.time()))
+                print(f"{t_begin:.2f} .. {time.time():.2f}  {label}: {table[-1]['tflops']:.1f} TFLOP/s", file=sys.stderr, flush=True)
+                time.sleep(1.0)
+            kernels["c4_energy_per_flop"] = table
+            del c4w
         if not ns.skip_cpu:
             from oracle import kernels as ok4
             a4c, b4c = a4[:1024].cpu(), b4.cpu()
@@ -495,6 +553,9 @@ def main():
         fl5 = sum(2 * m * n * k for m, n, k in dims)
         ms = timed(gg, steps=max(5, K // 5), warmup=max(2, W // 5))
         kernels["c5_grouped_gemm_f16"] = dict(ms=ms, tflops=fl5 / ms / 1e9, frac_mfma=fl5 / ms / 1e9 / MFMA_F16_PEAK_TFLOPS,
+                                              **({"achievable_tflops": kernels["mfma_ceiling_f16"]["tflops"],
+                                                  "frac_of_achievable": fl5 / ms / 1e9 / kernels["mfma_ceiling_f16"]["tflops"]}
+                                                 if "mfma_ceiling_f16" in kernels else {}),
                                               flop=fl5, problems=dims, rel_err_vs_fp32=rel)
         plan5 = (ctypes.c_int * 3)()
         runtime.call("lego_hip_grouped_gemm_f16_plan", sz, 8, plan5)

@@ -233,6 +233,13 @@ int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const 
                                    float* mean, float* rstd, int M, int N, float eps,
                                    int waves_per_row, void* stream);
 
+/* Tuning entry point: C = A * B (fp16, row-major, N and K multiples of 8, 16-byte aligned bases) on 256 x 256 tiles
+ * with the kernel chosen by the caller: variant 0 = what lego_hip_gemm_f16 launches for large products (four waves of
+ * 128 x 128, one per SIMD with 256 accumulator registers, v_mfma_f32_16x16x32_f16), 1 = the same workgroup with
+ * v_mfma_f32_32x32x16_f16, 2 = eight waves of 128 x 64, two per SIMD with 128 accumulator registers each
+ * (v_mfma_f32_32x32x16_f16).  Used by the benchmark to compare them.  No counterpart in the reference. */
+int lego_hip_gemm_f16_variant(const void* a, const void* b, void* c, int M, int N, int K, int variant, void* stream);
+
 /* Measurement aid: out[0..bytes) = in[0..bytes), 16 bytes per lane per access, bytes % 16 == 0.
  * No counterpart in the reference.  bench.py uses it as the same-run copy ceiling and the
  * profiles use it to calibrate the FETCH_SIZE / WRITE_SIZE counters at this access width. */
@@ -253,6 +260,22 @@ int lego_hip_copy16_stream(const void* in, void* out, unsigned long long bytes, 
  * bytes a multiple of the chunk.  bench.py times modes 0 and 1 on rotating 512 MiB buffers and derives from them
  * the rate that a kernel which reads and writes every byte once cannot pass on this part. */
 int lego_hip_hbm_probe(const void* in, void* out, unsigned long long bytes, int mode, int vectors_per_lane, void* stream);
+
+/* Measurement aid (no counterpart in the reference): what the matrix cores sustain when a kernel does nothing but
+ * issue MFMAs.  `workgroups` workgroups of four waves (one per SIMD, 256 accumulator registers each, the occupancy
+ * of the GEMM kernels); a wave loads sixteen 16-byte operand fragments per lane once (operands: workgroups * 64 KiB
+ * of 16-bit values, the caller's choice of distribution: the power a matrix core draws depends on its data) and
+ * runs `iters` rounds of MFMAs over a 128 x 128 block of accumulators: one MFMA per accumulator block and round,
+ * so a round is a k-step of the instruction's depth.
+ *   shape 0: v_mfma_f32_32x32x16_f16 (16 per round and wave: 2097152 flop per round and workgroup)
+ *   shape 1: v_mfma_f32_16x16x32_f16 (64 per round and wave: 4194304 flop per round and workgroup)
+ *   shape 2: v_mfma_f32_32x32x16_bf16 (the same bits read as bfloat16; flop as shape 0)
+ *   shape 3 / 4: the instructions of shapes 1 / 0 with two waves per SIMD (workgroups of eight waves with 128
+ *   accumulator registers each, a 128 x 64 block per wave: 4194304 / 2097152 flop per round and workgroup).
+ * sink: workgroups * 512 floats (a sum per lane, so that the work is not optimised away).  bench.py runs it with
+ * operands of the GEMM benchmark's distribution and reports the rate as what the socket's power limit leaves to
+ * an fp16 GEMM whose data movement costs nothing. */
+int lego_hip_mfma_probe(const void* operands, float* sink, int shape, int iters, int workgroups, void* stream);
 
 #ifdef __cplusplus
 }

@@ -65,9 +65,15 @@ ROWWISE_WIDE_TEAM_ABOVE_N, ROWWISE_WIDE_TEAM_FROM_M = 6144, 4096
 ROWWISE_MAX_N = rowwise.MAX_N
 GEMM = dict(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8)
 GEMM_SMALL_TILE = 128
+GEMM_WAVES_TWO_PER_SIMD = (2, 4)
 GEMM_SMALL_DTYPES = ("f16", "bf16", "bf16h")     # a 128-byte row of 8-bit elements is too short for their [k][n] rotation
 GEMM_SMALL_NT_ONLY = ("e4m3", "e5m2")             # ... so 8-bit operands get the small tile where both are k-major (A as given, B transposed)
 GEMM_DTYPES = ("f16", "bf16", "bf16h", "e4m3", "e5m2")     # bf16h: bfloat16 operands, fp16 result
+# The MFMA of the 256 x 256 tiles: v_mfma_f32_16x16x32 for 16-bit operands (the same matrix-core cycles per flop as
+# 32x32x16, but the socket's power limit leaves it a higher clock: a stream of nothing but MFMAs runs 1.95 against
+# 1.68 PFLOP/s, and the GEMM gains 3 to 7 %: 8192^3 1.29 -> 1.36, 4096^3 1.22 -> 1.31, 8192 x 8192 x 1024 1.12 -> 1.17
+# PFLOP/s); 32x32x64 for 8-bit operands.  The 128 x 128 tiles keep 32 x 32 blocks: their sums along K are laid out for them.
+GEMM_MFMA_BLOCK = {"f16": 16, "bf16": 16, "bf16h": 16, "e4m3": 32, "e5m2": 32}
 GEMM_BK = {"f16": 64, "bf16": 64, "bf16h": 64, "e4m3": 128, "e5m2": 128}   # 128 bytes of k per operand row in every case
 
 
@@ -109,7 +115,7 @@ def collect():
         for ta in (False, True):
             for tb in (False, True):
                 g, m_ = gemm.emit(**dict(GEMM, bk=GEMM_BK[dtype]), trans_a=ta, trans_b=tb, dtype=dtype,
-                                  with_grouped=dtype == "f16" and not (ta or tb),
+                                  block=GEMM_MFMA_BLOCK[dtype], with_grouped=dtype == "f16" and not (ta or tb),
                                   with_split=dtype == "f16" and not (ta or tb))
                 units.append(g)
                 if dtype == "f16":
@@ -125,6 +131,13 @@ def collect():
                     gs, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK[dtype], bm=GEMM_SMALL_TILE, bn=GEMM_SMALL_TILE),
                                       trans_a=ta, trans_b=tb, dtype=dtype, with_grouped=False)
                     units.append(gs)
+    # Two measured alternatives of the fp16 kernel, kept behind a tuning entry point so that the comparison can be
+    # repeated: 32 x 32 accumulator blocks (v_mfma_f32_32x32x16) with four waves of 128 x 128, and with eight waves of
+    # 128 x 64 per workgroup, two per SIMD with 128 accumulator registers each (a second wave to issue from while one
+    # waits).  8192^3: 1.29 and 1.28 PFLOP/s against 1.36.
+    g32, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK["f16"]), dtype="f16", with_grouped=False, suffix="_m32")
+    g8, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK["f16"], waves=GEMM_WAVES_TWO_PER_SIMD), dtype="f16", with_grouped=False)
+    units += [g32, g8]
     units.append(gemm.emit_any())
     lbs, mlb = layernorm_bwd.emit()
     units += lbs
@@ -206,6 +219,8 @@ def collect():
           "const int*, int, hipStream_t);",
           f"hipError_t lego_grouped_gemm_f16_t{GEMM_SMALL_TILE}x{GEMM_SMALL_TILE}_launch(const void* const*, "
           "const void* const*, void* const*, const int*, int, hipStream_t);",
+          "hipError_t lego_gemm_f16_nn_w2x4_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);",
+          "hipError_t lego_gemm_f16_nn_m32_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);",
           "hipError_t lego_gemm_any_launch(const void*, const void*, void*, int, int, int, int, int, int, int, hipStream_t);",
           "hipError_t lego_grouped_gemm_f16_split_launch(const void* const*, const void* const*, void* const*, "
           "const int*, int, int, hipStream_t);",

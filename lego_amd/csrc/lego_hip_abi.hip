@@ -84,6 +84,118 @@ __global__ void __launch_bounds__(256) lego_probe_copy_kernel(const u32x4* __res
   for (int u = 0; u < V; ++u) __builtin_nontemporal_store(v[u], out + base + u * 256);
 }
 
+// What the matrix cores sustain when nothing else happens: every wave of a workgroup of four (one per SIMD, 256
+// accumulator registers, as in the GEMM kernels) loads sixteen operand fragments once and then issues nothing but
+// MFMAs on them, a 128 x 128 block of accumulators per wave.  With random operands this is the rate the socket's
+// power limit leaves to a GEMM whose loads, LDS traffic and address arithmetic cost nothing.
+typedef _Float16 probe_half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 probe_bhalf8 __attribute__((ext_vector_type(8)));
+typedef float probe_float16 __attribute__((ext_vector_type(16)));
+typedef float probe_float4 __attribute__((ext_vector_type(4)));
+// The same with two waves per SIMD (workgroups of eight waves, 128 accumulator registers each, a 128 x 64 block):
+// whether a second wave to issue from changes what the pipe sustains.
+template <int SHAPE>      // 3: v_mfma_f32_16x16x32_f16 (8 x 4 blocks)  4: v_mfma_f32_32x32x16_f16 (4 x 2 blocks)
+__global__ void __launch_bounds__(512) lego_mfma_probe2_kernel(const probe_half8* __restrict__ operands, float* __restrict__ sink, unsigned iters)
+{
+  const probe_half8* mine = operands + (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x % 256) * 16;
+  probe_half8 fa[8], fb[4];
+#pragma unroll
+  for (int f = 0; f < 8; ++f) fa[f] = mine[f];
+#pragma unroll
+  for (int f = 0; f < 4; ++f) fb[f] = mine[8 + f];
+  float total = 0.0f;
+  if (SHAPE == 3) {
+    probe_float4 acc[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = probe_float4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (unsigned it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) total += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+  } else {
+    probe_float16 acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    for (unsigned it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) total += acc[i][j][r];
+  }
+  sink[static_cast<size_t>(blockIdx.x) * 512 + threadIdx.x] = total;
+}
+
+template <int SHAPE>      // 0: v_mfma_f32_32x32x16_f16 (4 x 4 blocks)  1: v_mfma_f32_16x16x32_f16 (8 x 8 blocks)  2: v_mfma_f32_32x32x16_bf16
+__global__ void __launch_bounds__(256) lego_mfma_probe_kernel(const probe_half8* __restrict__ operands, float* __restrict__ sink, unsigned iters)
+{
+  constexpr int T = SHAPE == 1 ? 8 : 4;
+  const probe_half8* mine = operands + (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 16;
+  probe_half8 fa[8], fb[8];
+#pragma unroll
+  for (int f = 0; f < 8; ++f) { fa[f] = mine[f]; fb[f] = mine[8 + f]; }
+  float total = 0.0f;
+  if (SHAPE == 1) {
+    probe_float4 acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[i][j] = probe_float4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (unsigned it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) total += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+  } else {
+    probe_float16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    for (unsigned it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < T; ++i)
+#pragma unroll
+        for (int j = 0; j < T; ++j) {
+          if (SHAPE == 0) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+          else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(probe_bhalf8, fb[j]), __builtin_bit_cast(probe_bhalf8, fa[i]), acc[i][j], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) total += acc[i][j][r];
+  }
+  sink[static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x] = total;
+}
+
 typedef unsigned u32x4w __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4w_any __attribute__((ext_vector_type(4), aligned(2)));     // the same 16 bytes at any 2-byte element
 
@@ -626,6 +738,15 @@ int lego_hip_gemm_fp8_ex(const void* a, const void* b, void* c, int M, int N, in
                  stream, LEGO_GEMM_BK_8BIT, 16);
 }
 
+int lego_hip_gemm_f16_variant(const void* a, const void* b, void* c, int M, int N, int K, int variant, void* stream)
+{
+  if (!usable(a) || !usable(b) || !usable(c) || M <= 0 || N <= 0 || K <= 0 || N % 8 || K % 8) return kInvalid;
+  if (variant == 0) return ok_or(lego_gemm_f16_nn_launch(a, b, c, M, N, K, 0, as_stream(stream)));
+  if (variant == 1) return ok_or(lego_gemm_f16_nn_m32_launch(a, b, c, M, N, K, 0, as_stream(stream)));
+  if (variant == 2) return ok_or(lego_gemm_f16_nn_w2x4_launch(a, b, c, M, N, K, 0, as_stream(stream)));
+  return kInvalid;
+}
+
 int lego_hip_gemm_f16_act(const void* a, const void* b, void* c, int M, int N, int K, int activation, void* stream)
 {
   return lego_hip_gemm_f16_ex(a, b, c, M, N, K, 0, 0, activation, stream);
@@ -954,6 +1075,20 @@ int lego_hip_hbm_probe(const void* in, void* out, unsigned long long bytes, int 
     else if (mode == 1) hipLaunchKernelGGL(lego_probe_write_kernel<4>, grid, block, 0, s, dst);
     else hipLaunchKernelGGL(lego_probe_copy_kernel<4>, grid, block, 0, s, src, dst);
   }
+  return ok_or(hipGetLastError());
+}
+
+int lego_hip_mfma_probe(const void* operands, float* sink, int shape, int iters, int workgroups, void* stream)
+{
+  if (!usable(operands) || !usable(sink) || shape < 0 || shape > 4 || iters <= 0 || workgroups <= 0) return kInvalid;
+  const dim3 grid(static_cast<unsigned>(workgroups)), block(256);
+  const probe_half8* src = static_cast<const probe_half8*>(operands);
+  hipStream_t s = as_stream(stream);
+  if (shape == 3) hipLaunchKernelGGL(lego_mfma_probe2_kernel<3>, grid, dim3(512), 0, s, src, sink, static_cast<unsigned>(iters));
+  else if (shape == 4) hipLaunchKernelGGL(lego_mfma_probe2_kernel<4>, grid, dim3(512), 0, s, src, sink, static_cast<unsigned>(iters));
+  else if (shape == 0) hipLaunchKernelGGL(lego_mfma_probe_kernel<0>, grid, block, 0, s, src, sink, static_cast<unsigned>(iters));
+  else if (shape == 1) hipLaunchKernelGGL(lego_mfma_probe_kernel<1>, grid, block, 0, s, src, sink, static_cast<unsigned>(iters));
+  else hipLaunchKernelGGL(lego_mfma_probe_kernel<2>, grid, block, 0, s, src, sink, static_cast<unsigned>(iters));
   return ok_or(hipGetLastError());
 }
 

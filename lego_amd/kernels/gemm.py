@@ -69,23 +69,27 @@ def lds_b_layout(bk, bn, period=4):
     return OrderBy(GenP((bk, bn), forward, backward)).TileBy([bk, bn])
 
 
-def lds_c_layout(rows, cols):
-    """A wave's block of C as fp16 in 8-byte chunks: ``row*(cols/4) + (chunk ^ (row % span))``,
-    ``span = min(32, cols/4)``.
+def lds_c_layout(rows, cols, block=32):
+    """A wave's block of C as fp16 in 8-byte chunks: ``row*(cols/4) + (chunk ^ key(row))``.
 
-    The accumulator layout makes 32 lanes store the same chunk of 32 consecutive rows; the
-    rotation spreads them over 32 different chunks of the 256-byte bank window (over 16, two
-    rows each, when a row has only 16 chunks)."""
+    32 x 32 accumulator blocks: 32 lanes store the same chunk of 32 consecutive rows; ``key = row % span``,
+    ``span = min(32, cols/4)``, spreads them over 32 different chunks of the 256-byte bank window (over 16, two rows
+    each, when a row has only 16 chunks).  16 x 16 blocks: the 32 lanes that are served together store two
+    neighbouring chunks of 16 consecutive rows; ``key = 2*(row % 16)`` spreads the rows over the 16 chunk pairs and
+    leaves a pair together and in order, so a 16-byte read-back needs no swap."""
     chunks = cols // 4
     span = min(32, chunks)
 
+    def key(row):
+        return row % span if block == 32 else 2 * (row % min(16, chunks // 2))
+
     def forward(rc):
         row, ch = rc
-        return row * chunks + BitXor(sp.sympify(ch), sp.sympify(row % span))
+        return row * chunks + BitXor(sp.sympify(ch), sp.sympify(key(row)))
 
     def backward(flat):
         row, p = flat // chunks, flat % chunks
-        return (row, BitXor(sp.sympify(p), sp.sympify(row % span)))
+        return (row, BitXor(sp.sympify(p), sp.sympify(key(row))))
 
     return OrderBy(GenP((rows, chunks), forward, backward)).TileBy([rows, chunks])
 
@@ -137,42 +141,46 @@ def lane_and_unit(expr, unit_vars, units, lane_vars, lane_values, stride):
 LAST_KTILE_RING = 8      # vectors a lane holds between reading them back from the staging block and storing them
 
 
-def last_ktile_schedule(TM, TN, NPH, WN):
+def last_ktile_schedule(TM, TN, NPH, WN, block=32, mps=1):
     """Slot schedule of a tile's last k-tile, in which the result leaves under the MFMAs.
 
-    The MFMAs go block row by block row (``i``), within a row k-step by k-step: slot ``i*SPR + ks*TN + j``,
-    ``SPR = TN*NPH``, so the accumulators of block row ``i`` are final when row ``i+1`` starts.  A slot also carries
-      loads   during row 0, every operand fragment the k-tile still needs, in the order of their first use (two
-              per slot at first): after row 0 no wave reads the operand buffers any more, and a barrier there
-              hands all of LDS to the staging of the results;
-      stage   during row ``i+1``, block row ``i`` converted and written to the wave's staging block, one unit =
-              four columns of a lane = (block, q) per ``4/NPH`` of a slot;
+    ``TM x TN`` accumulator blocks of ``block x block`` per wave, ``NPH`` k-steps per k-tile, ``mps`` MFMAs per slot (a
+    slot is what one scheduling fence encloses: 32 cycles of MFMA, so one 32x32x16 or two 16x16x32).  The MFMAs go
+    block row by block row (``i``), within a row k-step by k-step (MFMA ``i*TN*NPH + ks*TN + j``), so the accumulators
+    of block row ``i`` are final when row ``i+1`` starts.  A slot also carries
+      loads   during row 0, every operand fragment the k-tile still needs, in the order of their first use (the
+              first slots carry one more than the rest): after row 0 no wave reads the operand buffers any more, and
+              a barrier there hands all of LDS to the staging of the results;
+      stage   during row ``i+1``, block row ``i`` converted and written to the wave's staging block, a unit =
+              four columns of a lane = (block, q), spread evenly over the row's slots;
       rb, st  during row ``i+2``, the staged rows of block row ``i`` read back as 16-byte vectors (``rb``) and
-              stored to C two slots later (``st``: the LDS latency passes under two MFMAs).
+              stored to C two slots later (``st``: the LDS latency passes under the MFMAs between).
     What falls past the last row -- the staging of the last block row, the stores of the last two -- is the
-    ``tail``, in the same order without MFMAs.  Returns ``(slots, tail)``; a slot is a dict with the keys
-    ``mfma`` (i, j, ks), ``loads`` [(ks, f)], ``stage`` [(i, j, q)], ``rb`` [it], ``st`` [it], ``barrier``."""
-    assert 4 % NPH == 0 and WN % 16 == 0
-    SPR, U, IPR = TN * NPH, 4 // NPH, WN // 16
+    ``tail``, in the same order without MFMAs.  With more than one MFMA per slot the MFMAs are inline assembly whose
+    wait states the compiler does not know: the tail then holds a ``fence`` (a scheduling fence and the wait states
+    of the longest MFMA) in front of the first unit whose block took its last MFMA in the very last slot, so that
+    the read of that result cannot be issued too close behind it.  Returns ``(slots, tail)``; a slot is a dict with the keys
+    ``mfmas`` [(i, j, ks)], ``loads`` [(ks, f)], ``stage`` [(i, j, q)], ``rb`` [it], ``st`` [it], ``barrier``."""
+    Q = block * block // 64 // 4       # units of four accumulator registers per block
+    assert TN * NPH % mps == 0 and block * WN % 512 == 0
+    SPR, IPR = TN * NPH // mps, block * WN // 512      # slots, and read-backs (64 lanes x 16 bytes), per block row
     G = TM * SPR
-    slots = [dict(mfma=None, loads=[], stage=[], rb=[], st=[], barrier=False) for _ in range(G)]
+    slots = [dict(mfmas=[], loads=[], stage=[], rb=[], st=[], barrier=False) for _ in range(G)]
     for i in range(TM):
         for ks in range(NPH):
             for j in range(TN):
-                slots[i * SPR + ks * TN + j]["mfma"] = (i, j, ks)
+                slots[(i * TN * NPH + ks * TN + j) // mps]["mfmas"].append((i, j, ks))
     need = []                      # (ks, f): f < TM a fragment of A's block row f, else of B's block column f - TM
     for ks in range(1, NPH):
         need += [(ks, 0)] + [(ks, TM + j) for j in range(TN)]
     for i in range(1, TM):
         need += [(ks, i) for ks in range(1, NPH)]
-    doubles = max(0, len(need) - SPR)
-    assert doubles <= SPR
     at = 0
-    for s_ in range(SPR):
-        for _ in range(2 if s_ < doubles else 1):
-            if at < len(need):
-                slots[s_]["loads"].append(need[at])
-                at += 1
+    for s_ in range(SPR):      # spread over the slots of row 0, the first slots one more than the rest
+        for _ in range(len(need) // SPR + (1 if s_ < len(need) % SPR else 0)):
+            slots[s_]["loads"].append(need[at])
+            at += 1
+    assert at == len(need)
     slots[SPR - 1]["barrier"] = True
     late = []                      # (global slot, order, kind, payload) of what falls past the last MFMA
     def put(g, kind, payload):
@@ -181,8 +189,8 @@ def last_ktile_schedule(TM, TN, NPH, WN):
         else:
             late.append((g, len(late), kind, payload))
     for r in range(TM):
-        for u, (j, q) in enumerate((j, q) for j in range(TN) for q in range(4)):
-            put((r + 1) * SPR + u // U, "stage", (r, j, q))
+        for u, (j, q) in enumerate((j, q) for j in range(TN) for q in range(Q)):
+            put((r + 1) * SPR + u * SPR // (TN * Q), "stage", (r, j, q))
         for m in range(IPR):
             g = (r + 2) * SPR + m * SPR // IPR
             put(g, "rb", r * IPR + m)
@@ -196,7 +204,13 @@ def last_ktile_schedule(TM, TN, NPH, WN):
     early = [it for kind, it in ordered if kind == "rb" and it // IPR < TM - 1]
     assert len(early) <= LAST_KTILE_RING
     tail += [("rb", it) for it in early]
-    tail += [(kind, u) for kind, u in ordered if kind == "stage"]
+    fenced = False
+    for kind, u in ordered:
+        if kind == "stage":
+            if mps > 1 and not fenced and (u[0] * TN * NPH + (NPH - 1) * TN + u[1]) // mps == G - 1:
+                tail.append(("fence", None))
+                fenced = True
+            tail.append((kind, u))
     tail += [("st", it) for it in early]
     fresh = [it for kind, it in ordered if kind == "rb" and it // IPR == TM - 1]
     for first in range(0, len(fresh), LAST_KTILE_RING):
@@ -205,8 +219,9 @@ def last_ktile_schedule(TM, TN, NPH, WN):
     return slots, tail
 
 
-def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped, dtype):
-    """Everything the templates need for one tile shape."""
+def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped, dtype, block=32, suffix=""):
+    """Everything the templates need for one tile shape.  ``block``: 32 = v_mfma_f32_32x32x16 (x64 for 8-bit operands),
+    16 = v_mfma_f32_16x16x32 (16-bit operands), the side of an accumulator block."""
     # element type, bytes per element, k-depth of one MFMA, result type; the 8-bit types are the
     # OCP formats of v_mfma_f32_32x32x64_f8f6f4 (format code 0 = e4m3, 1 = e5m2)
     # "bf16h": bfloat16 operands with the fp16 result that the reference's matmul stores whatever its
@@ -217,10 +232,14 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
                                    "e5m2": ("unsigned char", 1, 64, "_Float16")}[dtype]
     EPC = 16 // esize                      # elements per 16-byte chunk
     assert not (with_grouped and dtype != "f16"), "the grouped kernel is built for fp16 only"
+    assert block in (32, 16) and (block == 32 or esize == 2)
+    if block == 16:
+        mfma_k = 32
+    MPS = 32 // block                      # MFMAs per scheduling slot: a slot is 32 cycles of matrix-core work
     WAVES_M, WAVES_N = waves
     THREADS = 64 * WAVES_M * WAVES_N
     WM, WN = bm // WAVES_M, bn // WAVES_N
-    TM, TN = WM // 32, WN // 32
+    TM, TN = WM // block, WN // block
     A_ITERS = bm * bk // EPC // THREADS
     B_ITERS = bk * bn // EPC // THREADS
     assert bm * bk // EPC % THREADS == 0 and bk * bn // EPC % THREADS == 0 and bk % mfma_k == 0
@@ -230,7 +249,7 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
     # next phase and the memory->LDS instructions are spread evenly over them (for the 256x256
     # tile: a fragment on every even slot, a copy on every odd one).  The copies of a k-tile go into
     # the phase after the barrier (the first DMA_LAST) and the phase that follows it (the rest).
-    SLOTS, FRAGS, COPIES = TM * TN, TM + TN, A_ITERS + B_ITERS
+    SLOTS, FRAGS, COPIES = TM * TN // MPS, TM + TN, A_ITERS + B_ITERS
     assert NPH >= 2 and NPH % 2 == 0, "fragments are double buffered by phase parity"
     # With two phases per k-tile (8-bit operands) the phase before the barrier is the only one a copy issued in it
     # would have to land in: all copies go behind the barrier, one per slot, and have the whole next phase
@@ -251,7 +270,7 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
         load_slots[f * SLOTS // FRAGS].append(f)
     dma_last, dma_first = spread(0, DMA_LAST), spread(DMA_LAST, COPIES - DMA_LAST)
     none = [[] for _ in range(SLOTS)]
-    last_slots, last_tail = last_ktile_schedule(TM, TN, NPH, WN)
+    last_slots, last_tail = last_ktile_schedule(TM, TN, NPH, WN, block, MPS)
 
     M, N, K = size("M"), size("N"), size("K")
     npm, npn, per_xcd, group_m = size("num_pid_m"), size("num_pid_n"), size("wg_per_xcd"), size("GM")
@@ -279,6 +298,9 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
            wm: (0, WAVES_M), wn: (0, WAVES_N), l32: (0, 32), lhi: (0, 2), l16: (0, 16),
            lgrp: (0, 4), ks: (0, NPH), cr: (0, bm), cc: (0, bn), pid_m: (0, M / bm),
            pid_n: (0, N / bn), k: (0, K / bk)}
+    # the lane's row (column) of an MFMA operand block and its k block: lane % 32 and lane / 32 for 32 x 32 blocks,
+    # lane % 16 and lane / 16 for 16 x 16 ones
+    lrow, lk = (l32, lhi) if block == 32 else (l16, lgrp)
 
     def chunk_walk(expr, n_iters):
         """``expr`` (a function of the lane ``t`` and the chunk counter ``it``) as
@@ -299,7 +321,7 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
                         raise ValueError("chunk offsets are not affine in the instruction counter")
         return at[0], step
 
-    Cs_L = lds_c_layout(WM, WN)
+    Cs_L = lds_c_layout(WM, WN, block)
     cp = idx("cp")
     rng.update({cr: (0, WM), cp: (0, WN // 8)})
     lane_o = idx("lane")
@@ -310,18 +332,24 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
 
     # The staging block of the results, as the last k-tile's schedule addresses it (elements of the result type):
     # a unit (i, j, q) writes four columns of a lane, a read-back `it` fetches 16 bytes of row 4*it + lane/16.
-    stage_e = tidy(4 * Cs_L[i * 32 + l32, j * 8 + q * 2 + lhi], rng)
-    back_e = (tidy(4 * Cs_L[cr, 2 * cp], rng) - 4 * (cr % 2)).subs({cr: c_out[0], cp: c_out[1]})
-    lanes_mfma = [(a_, b_) for a_ in range(32) for b_ in range(2)]
-    stage_lane, stage_ax = lane_and_unit(stage_e, (i, j, q), [(a_, b_, c_) for a_ in range(TM) for b_ in range(TN) for c_ in range(4)],
-                                         (l32, lhi), lanes_mfma, 32 * WN)
+    # (a lane of a 32 x 32 block holds columns 8q + 4*(lane/32) .. +3 of row lane%32 in registers 4q..4q+3, a lane of a
+    # 16 x 16 block columns 4*(lane/16) .. +3 of row lane%16 in its four registers)
+    if block == 32:
+        stage_e = tidy(4 * Cs_L[i * 32 + l32, j * 8 + q * 2 + lhi], rng)
+        back_e = (tidy(4 * Cs_L[cr, 2 * cp], rng) - 4 * (cr % 2)).subs({cr: c_out[0], cp: c_out[1]})
+    else:
+        stage_e = tidy(4 * Cs_L[i * 16 + l16, j * 4 + lgrp], rng) + 0 * q
+        back_e = tidy(4 * Cs_L[cr, 2 * cp], rng).subs({cr: c_out[0], cp: c_out[1]})     # pairs stay in order: no swap
+    lanes_mfma = [(a_, b_) for a_ in range(block) for b_ in range(64 // block)]
+    stage_lane, stage_ax = lane_and_unit(stage_e, (i, j, q), [(a_, b_, c_) for a_ in range(TM) for b_ in range(TN) for c_ in range(block * block // 256)],
+                                         (lrow, lk), lanes_mfma, block * WN)
     n_its = WM * WN // 8 // 64
     back_lane, back_ax = lane_and_unit(back_e, (it,), [(a_,) for a_ in range(n_its)], (lane_o,), [(a_,) for a_ in range(64)], 512)      # a wave instruction moves 64 x 8 elements
 
     def with_constants(kind, payload):
         if kind == "stage":
             return tuple(payload) + stage_ax[tuple(payload)]
-        return (payload,) + back_ax[(payload,)] if kind == "rb" else payload
+        return (payload,) + back_ax[(payload,)] if kind == "rb" else payload      # "st": the vector, "fence": nothing
     for slot_ in last_slots:
         slot_["stage"] = [with_constants("stage", u) for u in slot_["stage"]]
         slot_["rb"] = [with_constants("rb", u) for u in slot_["rb"]]
@@ -345,7 +373,7 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
         comes from, the k-tile stride, and the text that reads one MFMA fragment."""
         kmajor = a_kmajor if role == "a" else b_kmajor
         rows, tile_id = (bm, pid_m) if role == "a" else (bn, pid_n)
-        wave_off, sub = (wm * WM + i * 32, i) if role == "a" else (wn * WN + j * 32, j)
+        wave_off, sub = (wm * WM + i * block, i) if role == "a" else (wn * WN + j * block, j)
         n_iters = A_ITERS if role == "a" else B_ITERS
 
         def glob(row_e, kk_e):   # offset of element (row, kk) of k-tile k of this operand's tile
@@ -356,9 +384,11 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
             r_e, ch_e = (tidy(e, slot_rng) for e in lds.inv(slot))
             full = tidy(glob(row, ch * EPC), rng)
             placed = full.subs({row: r_e, ch: ch_e})
-            # a lane's mfma_k/2 k-values of row l32: one 16-byte chunk (2-byte elements) or two
-            n_ch = mfma_k // 2 // EPC
-            chunks = [code(tidy(EPC * lds[wave_off + l32, (ks * 2 + lhi) * n_ch + c], rng)) for c in range(n_ch)]
+            # a lane's k-values of its row of the block (mfma_k/2 of them for 32-row blocks, mfma_k/4 for 16-row ones): one
+            # 16-byte chunk (2-byte elements) or two
+            k_blocks = 64 // block
+            n_ch = mfma_k // k_blocks // EPC
+            chunks = [code(tidy(EPC * lds[wave_off + lrow, (ks * k_blocks + lk) * n_ch + c], rng)) for c in range(n_ch)]
             if esize == 2:
                 frag = "*reinterpret_cast<const half8*>(%ss + (%s))" % (role, chunks[0])
             else:
@@ -368,7 +398,11 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
             kr_e, col_e = (tidy(e, slot_rng) for e in lds.inv(EPC * slot))
             full = tidy(glob(EPC * ch, kr), rng)    # here `ch` counts 16-byte chunks along the row
             placed = full.subs({kr: kr_e, ch: tidy(col_e / EPC, slot_rng)})
-            if esize == 2:
+            if esize == 2 and block == 16:
+                # (16-column blocks: the four lane groups are the four k blocks of eight)
+                frag_k = [ks * 32 + lgrp * 8 + h * 4 + l16 // 4 for h in (0, 1)]
+                frag_c = wave_off + 4 * (l16 % 4)
+            elif esize == 2:
                 # a transposing read hands lane 16g+i four consecutive k of column i of group g's
                 # 16 columns; source lane s supplies k-row s/4 and columns 4*(s%4)..+3
                 frag_k = [ks * 16 + (lgrp // 2) * 8 + h * 4 + l16 // 4 for h in (0, 1)]
@@ -395,7 +429,7 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
                 f"{role}_frag_code": frag}
 
     variant = ("t" if trans_a else "n") + ("t" if trans_b else "n")
-    tag = "" if (bm, bn) == (256, 256) else f"_t{bm}x{bn}"
+    tag = ("" if (bm, bn) == (256, 256) else f"_t{bm}x{bn}") + ("" if tuple(waves) == (2, 2) else f"_w{WAVES_M}x{WAVES_N}") + suffix
     chunk_params = dict(WAVES=WAVES, variant=variant, tag=tag, with_grouped=with_grouped, **operand("a"), **operand("b"))
 
     params = dict(
@@ -415,11 +449,12 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
         # offset of a chunk = tile base (uniform) + position inside k-tile 0 (per lane) + k * step
         **chunk_params,
         # accumulator -> staging: row i*32 + l32, 8-byte chunk (j*32 + q*8 + lhi*4)/4 of the wave's block
-        c_stage_store=code(tidy(4 * Cs_L[i * 32 + l32, j * 8 + q * 2 + lhi], rng)),
+        c_stage_store=code(stage_e),
         # staging -> memory: lane reads the pair of chunks (2p, 2p+1) of row cr; the XOR keeps a
-        # pair together and swaps its halves on odd rows
+        # pair together and (32 x 32 blocks) swaps its halves on odd rows
         c_out_row=code(c_out[0]), c_out_pair=code(c_out[1]),
-        c_stage_load=code(tidy(4 * Cs_L[cr, 2 * cp], rng) - 4 * (cr % 2)),
+        c_stage_load=code(tidy(4 * Cs_L[cr, 2 * cp], rng) - (4 * (cr % 2) if block == 32 else 0)),
+        BLOCK=block, MPS=MPS, ACC_REGS=block * block // 64, SWAP_ODD_ROWS=block == 32,
         c_goff=code(tidy(C_L[pid_m, pid_n, wm * WM + cr, wn * WN + 8 * cp], rng)),
         c_stage_lane=code(stage_lane), c_back_lane=code(back_lane),
         c_wave=code(c_wave_e), c_lane=code(c_lane_e), c_it_step=code(c_it_e),
@@ -452,19 +487,21 @@ def split_order(split, wg):
 
 
 def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, trans_b=False, with_grouped=True,
-         dtype="f16", with_split=False, with_splitk=False):
+         dtype="f16", with_split=False, with_splitk=False, block=32, suffix=""):
     """One translation unit: the GEMM kernel of one operand layout and element type on ``bm x bn``
     tiles, with ``with_grouped`` the grouped kernel on the same tiles, and with ``with_split`` a
     second grouped kernel that gives the last tiles of its launch to two workgroups each, as
     halves of ``bm/2 x bn`` (the tail of a launch whose last round of whole tiles would leave most
-    CUs idle)."""
-    params = _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped, dtype)
+    CUs idle).  ``block``: the side of the MFMA's accumulator block (see ``_tile_params``); ``suffix`` goes behind
+    the names of the file and the launchers (a second build of one shape)."""
+    assert not (with_splitk and block != 32), "partial sums along K are laid out for 32 x 32 accumulator blocks"
+    params = _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped, dtype, block, suffix)
     ns = f"t{bm}x{bn}"
     tiles = [dict(ns=ns, text=template("gemm_tile.hip.j2").render(**params))]
     params.update(main_ns=ns, with_split=with_split, with_splitk=with_splitk)
     if with_split:
         assert with_grouped
-        half = _tile_params(bm // 2, bn, bk, waves, max_group_m, trans_a, trans_b, True, dtype)
+        half = _tile_params(bm // 2, bn, bk, waves, max_group_m, trans_a, trans_b, True, dtype, block)
         hns = f"t{bm // 2}x{bn}"
         tiles.append(dict(ns=hns, text=template("gemm_tile.hip.j2").render(**half)))
         split, swg, ti, hf = size("split"), idx("swg"), idx("pid_m"), idx("half")

@@ -30,6 +30,7 @@ SIGNATURES = {
     "lego_hip_layernorm_fwd_f16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                    _c_int, _c_int, _c_float, _c_void_p],
     "lego_hip_gemm_f16": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    "lego_hip_gemm_f16_variant": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "lego_hip_gemm_f16_act": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "lego_hip_gemm_f16_ex": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                              _c_void_p],
@@ -63,6 +64,7 @@ SIGNATURES = {
     "lego_hip_copy16": [_c_void_p, _c_void_p, ctypes.c_ulonglong, _c_void_p],
     "lego_hip_copy16_stream": [_c_void_p, _c_void_p, ctypes.c_ulonglong, _c_void_p],
     "lego_hip_hbm_probe": [_c_void_p, _c_void_p, ctypes.c_ulonglong, _c_int, _c_int, _c_void_p],
+    "lego_hip_mfma_probe": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
 }
 
 _lib = None

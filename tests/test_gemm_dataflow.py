@@ -10,8 +10,9 @@ lane/element rule measured on gfx950:
 * ``ds_read_b64_tr_b8``: lane ``i`` receives byte ``i % 8`` of source lanes ``i//8 + 2*j``,
   ``j = 0..7``.
 
-Expected: lane ``l`` of an MFMA operand holds row/column ``l % 32`` and the ``k``-values
-``(l // 32) * kk .. + kk - 1`` of the k-step, ``kk`` = 8 (16-bit) or 32 (8-bit), in order.
+Expected: lane ``l`` of an MFMA operand holds row/column ``l % block`` and the ``k``-values
+``(l // block) * kk .. + kk - 1`` of the k-step, ``kk`` = 8 (16-bit) or 32 (8-bit), in order; ``block`` = 32 for
+the 32x32 MFMAs (a k-step of 2 kk), 16 for v_mfma_f32_16x16x32 (a k-step of 4 kk).
 """
 import re
 
@@ -47,11 +48,12 @@ def _args(call):
     return out + [cur]
 
 
-@pytest.mark.parametrize("dtype,bk,tile", [("f16", 64, 256), ("e5m2", 128, 256), ("f16", 64, 128)])
+@pytest.mark.parametrize("dtype,bk,tile,block", [("f16", 64, 256, 32), ("f16", 64, 256, 16), ("e5m2", 128, 256, 32),
+                                                 ("f16", 64, 128, 32)])
 @pytest.mark.parametrize("variant", ["nn", "tt"])
-def test_fragments_receive_the_right_elements(dtype, bk, tile, variant):
+def test_fragments_receive_the_right_elements(dtype, bk, tile, block, variant):
     ta, tb = variant[0] == "t", variant[1] == "t"
-    unit, _ = gemm.emit(bm=tile, bn=tile, bk=bk, trans_a=ta, trans_b=tb, with_grouped=False, dtype=dtype)
+    unit, _ = gemm.emit(bm=tile, bn=tile, bk=bk, trans_a=ta, trans_b=tb, with_grouped=False, dtype=dtype, block=block)
     text = unit.text
     esize = 2 if dtype == "f16" else 1
     epc = 16 // esize                       # elements per 16-byte chunk
@@ -83,11 +85,12 @@ def test_fragments_receive_the_right_elements(dtype, bk, tile, variant):
         assert (lds >= 0).all() and len(set(lds.tolist())) == tile * bk    # the whole tile, once
         # --- what the fragment reads hand to the lanes
         frag = _grab(text, r"f%s\[BUF\]\[%s\] = (.*?); \}" % (role, "i" if role == "a" else "j"))
-        for ks in range(bk // (2 * kk)):
-            for sub in range(tile // 64):
+        groups = 64 // block                        # lane groups of an operand, kk k-values each
+        for ks in range(bk // (groups * kk)):
+            for sub in range(tile // 2 // block):
                 for w in range(2):
                     env0 = dict(ks=ks, i=sub, j=sub, wm=w, wn=w)
-                    want_row0 = w * (tile // 2) + sub * 32
+                    want_row0 = w * (tile // 2) + sub * block
 
                     def addr(expr, lane):
                         env = dict(env0, l32=lane % 32, lhi=lane // 32, l16=lane % 16, lgrp=lane // 16)
@@ -116,8 +119,8 @@ def test_fragments_receive_the_right_elements(dtype, bk, tile, variant):
                                     assert p0 % per == 0
                                     got[lane, r * per + jj] = lds[p0 + i_ % per]
                     for lane in range(64):
-                        row = want_row0 + lane % 32
-                        k0 = ks * 2 * kk + (lane // 32) * kk
+                        row = want_row0 + lane % block
+                        k0 = ks * groups * kk + (lane // block) * kk
                         assert got[lane].tolist() == [row * bk + k0 + x for x in range(kk)], (role, ks, sub, w, lane)
 
 

@@ -7,38 +7,59 @@ import pytest
 
 from lego_amd.kernels import gemm
 
-SHAPES = [(4, 4, 4, 128), (2, 2, 4, 64), (2, 4, 4, 128), (4, 4, 2, 128), (2, 2, 2, 64)]      # TM, TN, NPH, WN of every tile built
+# TM, TN, NPH, WN, block, MFMAs per slot of every tile built: 32x32x16 (and 32x32x64 for 8-bit) blocks one per slot,
+# 16x16x32 blocks two per slot
+SHAPES = [(4, 4, 4, 128, 32, 1), (2, 2, 4, 64, 32, 1), (2, 4, 4, 128, 32, 1), (4, 4, 2, 128, 32, 1), (2, 2, 2, 64, 32, 1),
+          (4, 2, 4, 64, 32, 1), (8, 8, 2, 128, 16, 2), (4, 8, 2, 128, 16, 2), (4, 4, 2, 64, 16, 2)]
 
 
-@pytest.mark.parametrize("TM,TN,NPH,WN", SHAPES)
-def test_last_ktile_schedule_is_a_valid_order(TM, TN, NPH, WN):
-    slots, tail = gemm.last_ktile_schedule(TM, TN, NPH, WN)
-    assert len(slots) == TM * TN * NPH
-    rows_per_it = WN // 16                                   # read-backs per block row of 32 rows
+@pytest.mark.parametrize("TM,TN,NPH,WN,block,mps", SHAPES)
+def test_last_ktile_schedule_is_a_valid_order(TM, TN, NPH, WN, block, mps):
+    slots, tail = gemm.last_ktile_schedule(TM, TN, NPH, WN, block, mps)
+    assert len(slots) == TM * TN * NPH // mps
+    rows_per_it = block * WN // 512                          # read-backs per block row
+    units_per_block = block * block // 256
     have = {(0, f) for f in range(TM + TN)}                  # fragments of k-step 0 arrive with the tile
     done = {}                                                # block -> k-steps summed
     events = []
+    final_slot = {}
     barrier_at = None
     for g, slot in enumerate(slots):
         for ks, f in slot["loads"]:
             assert barrier_at is None, "a fragment read after the operand buffers were handed over"
             assert 0 < ks < NPH and 0 <= f < TM + TN and (ks, f) not in have
             have.add((ks, f))
-        i, j, ks = slot["mfma"]
-        assert (ks, i) in have and (ks, TM + j) in have, f"slot {g}: fragment not read yet"
-        assert done.get((i, j), 0) == ks                     # k-steps of a block in order
-        done[(i, j)] = ks + 1
+        assert len(slot["mfmas"]) == mps
+        for i, j, ks in slot["mfmas"]:
+            assert (ks, i) in have and (ks, TM + j) in have, f"slot {g}: fragment not read yet"
+            assert done.get((i, j), 0) == ks                 # k-steps of a block in order
+            done[(i, j)] = ks + 1
+            final_slot[(i, j)] = g
         for i2, j2, q in slot["stage"]:
             assert barrier_at is not None and done.get((i2, j2), 0) == NPH, f"slot {g}: block ({i2}, {j2}) staged early"
+            # (a whole slot of MFMAs lies between an inline-assembly MFMA and the read of its result)
+            assert mps == 1 or g - final_slot[(i2, j2)] >= 2
             events.append(("stage", (i2, j2, q)))
         events += [("rb", it) for it in slot["rb"]] + [("st", it) for it in slot["st"]]
         if slot["barrier"]:
             assert barrier_at is None
             barrier_at = g
     assert len(have) == NPH * (TM + TN) and all(v == NPH for v in done.values()) and len(done) == TM * TN
+    # MFMAs as inline assembly (more than one per slot): a fence (with the wait states of an MFMA) stands between
+    # the last slot and the first read of one of its results
+    last_slot_blocks = {(i, j) for i, j, ks in slots[-1]["mfmas"] if ks == NPH - 1}
+    staged_in_tail = [u[:2] for kind, u in tail if kind == "stage"]
+    if mps > 1:
+        at = [kind for kind, u in tail].index("fence")
+        before = [u[:2] for kind, u in tail[:at] if kind == "stage"]
+        assert not last_slot_blocks & set(before)
+        assert last_slot_blocks <= set(staged_in_tail)
+    else:
+        assert all(kind != "fence" for kind, u in tail)
+    tail = [(kind, u) for kind, u in tail if kind != "fence"]
     events += [(kind, tuple(u) if kind == "stage" else u) for kind, u in tail]
     units = [u for kind, u in events if kind == "stage"]
-    assert sorted(units) == sorted((i, j, q) for i in range(TM) for j in range(TN) for q in range(4))
+    assert sorted(units) == sorted((i, j, q) for i in range(TM) for j in range(TN) for q in range(units_per_block))
     for kind in ("rb", "st"):
         assert sorted(u for k, u in events if k == kind) == list(range(TM * rows_per_it))
     in_flight = {}
