@@ -250,6 +250,44 @@ def generate():
     return paths
 
 
+# Instructions that must lie between an MFMA written as inline assembly and the first other instruction that reads
+# its result: the compiler inserts the wait states of MFMAs it knows (at most 19, for the sixteen-pass ones) but does
+# not look into inline assembly.  The 16x16x32 MFMA takes four passes; the kernels built keep 23 and more.
+ASM_MFMA_MIN_DISTANCE = 16
+
+
+def asm_mfma_read_distance(assembly: str):
+    """Smallest number of instructions, per function of a gfx950 assembly listing, between an MFMA and the next
+    instruction other than an MFMA that names one of the accumulation registers it writes (``a7`` or a range
+    ``a[4:7]``), counted along the listing: ``{function: (distance, register, instruction)}``.  Functions in which
+    no MFMA result is read back are left out."""
+    import re
+    out, name, last, count = {}, None, {}, 0
+    for line in assembly.split("\n"):
+        text = line.strip()
+        m = re.match(r"^([A-Za-z_][\w$.]*):", line)
+        if m and not text.startswith("."):
+            name, last, count = m.group(1), {}, 0
+            continue
+        if not text or text[0] in ";." or text.endswith(":"):
+            continue
+        count += 1
+        m = re.match(r"v_mfma\S+\s+a\[(\d+):(\d+)\]", text)
+        if m:
+            for r in range(int(m.group(1)), int(m.group(2)) + 1):
+                last[r] = count
+            continue
+        regs = [int(r) for r in re.findall(r"\ba(\d+)\b", text)]
+        for lo, hi in re.findall(r"\ba\[(\d+):(\d+)\]", text):
+            regs += range(int(lo), int(hi) + 1)
+        for r in regs:
+            if r in last and text.split()[0] not in ("v_accvgpr_write_b32", "v_accvgpr_mov_b32"):
+                found = (count - last[r], r, text.split()[0])
+                if name not in out or found < out[name]:
+                    out[name] = found
+    return out
+
+
 def _compile(src: Path, incremental: bool = False) -> Path:
     obj = OBJ_DIR / (src.stem + ".o")
     if incremental and obj.exists():
@@ -260,9 +298,21 @@ def _compile(src: Path, incremental: bool = False) -> Path:
         if obj.stat().st_mtime > newest:
             return obj
     cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", str(ROOT / "include"), "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
+    asm_mfma = "asm volatile(\"v_mfma" in src.read_text()
+    if asm_mfma:       # keep the device assembly beside the object and check what the compiler cannot
+        cmd.insert(1, "-save-temps=obj")
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src.name}:\n{res.stderr}")
+    if asm_mfma:
+        listing = OBJ_DIR / f"{src.stem}-hip-amdgcn-amd-amdhsa-gfx950.s"
+        close = {f: d for f, d in asm_mfma_read_distance(listing.read_text()).items() if d[0] < ASM_MFMA_MIN_DISTANCE}
+        for temp in [*OBJ_DIR.glob(f"{src.stem}-h*"), *OBJ_DIR.glob(f"{src.stem}.hip-*")]:
+            temp.unlink()
+        if close:
+            obj.unlink()
+            raise RuntimeError(f"{src.name}: an accumulator is read within {ASM_MFMA_MIN_DISTANCE} instructions of "
+                               f"the inline-assembly MFMA that writes it: {close}")
     return obj
 
 

@@ -98,3 +98,19 @@ def test_staging_offsets_split_into_lane_and_unit_constants():
                 assert cexpr(p["c_stage_load"], cr=cr, cp=cp) == add + (cexpr(p["c_back_lane"], lane=lane) ^ xor)
                 seen += 1
     assert seen > 300
+
+
+def test_build_check_finds_an_accumulator_read_close_behind_an_inline_assembly_mfma():
+    """The build reads the device assembly of every unit whose MFMAs are inline assembly: the checker behind it, on
+    two listings -- a result read three instructions after its MFMA, and one read after twenty."""
+    from lego_amd import build
+    mfma = "\tv_mfma_f32_16x16x32_f16 a[4:7], v[2:5], v[6:9], a[4:7]\n"
+    other = "\tv_add_u32_e32 v1, v2, v3\n"
+    head = "\t.text\nkernel_a:\n; %bb.0:\n"
+    close = head + mfma + other * 2 + "\tv_accvgpr_read_b32 v10, a5\n\ts_endpgm\n"
+    far = head + mfma + "\tv_mfma_f32_16x16x32_f16 a[0:3], v[2:5], v[6:9], a[0:3]\n" + other * 19 + \
+        "\tv_accvgpr_read_b32 v10, a[4:5]\n\ts_endpgm\nkernel_b:\n" + mfma + "\ts_endpgm\n"
+    assert build.asm_mfma_read_distance(close) == {"kernel_a": (3, 5, "v_accvgpr_read_b32")}
+    found = build.asm_mfma_read_distance(far)
+    assert found == {"kernel_a": (21, 4, "v_accvgpr_read_b32")}      # kernel_b reads nothing back
+    assert found["kernel_a"][0] >= build.ASM_MFMA_MIN_DISTANCE > 3
