@@ -211,11 +211,18 @@ def main():
         rot = rotating(lambda: (torch.rand(n1, n1, device=dev), torch.empty(n1, n1, device=dev)),
                        lambda s: runtime.call("lego_hip_transpose_f32", p(s[0]), p(s[1]), n1, n1, stream),
                        1 << 30, b1)
+        # a launch this short pays its ramp: the same bytes through a plain copy (one 16-byte vector per lane), same pool
+        rot_copy = rotating(lambda: (torch.rand(n1, n1, device=dev), torch.empty(n1, n1, device=dev)),
+                            lambda s: runtime.call("lego_hip_hbm_probe", p(s[0]), p(s[1]), n1 * n1 * 4, 2, 1, stream),
+                            1 << 30, b1)
         kernels["c1_transpose_f32_4096"] = dict(ms_hot=hot, gbs_hot=b1 / hot / 1e6, ms=rot, gbs=b1 / rot / 1e6,
                                                 frac_hbm=b1 / rot / 1e6 / HBM_PEAK_GBS, bytes=b1,
                                                 achievable_gbs=achievable, frac_of_achievable=b1 / rot / 1e6 / achievable,
+                                                plain_copy_same_bytes_gbs=b1 / rot_copy / 1e6,
+                                                frac_of_plain_copy=rot_copy / rot,
                                                 parity="bit-exact",
-                                                note="gbs = rotating buffers (1 GiB pool); gbs_hot = cache resident")
+                                                note="gbs = rotating buffers (1 GiB pool); gbs_hot = cache resident; "
+                                                     "plain_copy_same_bytes = a copy kernel over the same 2 x 64 MiB")
         if not ns.skip_cpu:
             from lego_amd.kernels.transpose import python_offsets
             from oracle import cpu_path

@@ -226,6 +226,13 @@ int lego_hip_grouped_gemm_f16_plan(const int* sizes3, int groups, int* plan3);
 int lego_hip_grouped_gemm_f16_split(const void* const* a, const void* const* b, void* const* c,
                                     const int* sizes3, int groups, int split_tiles, void* stream);
 
+/* Tuning entry points: the transposes with the tiling chosen by the caller, by its place in the library's list of
+ * tilings for the element type (lego_amd/build.py, TRANSPOSE; 0 = the first).  Invalid value if the list has no such
+ * entry or the shape is not one that tiling takes (whole windows of macro tiles for the first ones); bases 16-byte
+ * aligned.  Used by the benchmark to compare tilings on one shape.  No counterpart in the reference. */
+int lego_hip_transpose_f32_tiling(const void* in, void* out, int rows, int cols, int tiling, void* stream);
+int lego_hip_transpose_f16_tiling(const void* in, void* out, int rows, int cols, int tiling, void* stream);
+
 /* Tuning entry points: as above, with the launch shape chosen by the caller
  * (waves_per_row in {1, 2, 4, 8, 16}; N a multiple of 8 and at most 8192 * waves_per_row, 16384 for 4 and 8).  Used by the benchmark to compare variants. */
 int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per_row, void* stream);

@@ -27,21 +27,31 @@ OBJ_DIR = LIB_DIR / "obj"
 # Per element type, in order of preference: the fastest tiling for shapes that its windows
 # divide (then the same in smaller windows), a wide macro tile in skewed ("diag") order, a 64x64 one for shapes the wide tile
 # does not divide, and the wide tile with edge tests for shapes in whole 16-byte vectors.
+# The tilings with edge tests run their tiles in strips eight tile columns wide and load with plain (cached) loads:
+# when a row is not a whole number of 128-byte lines the row segments of neighbouring tiles share lines, and a
+# tile's neighbours on all four sides then run on the same XCD at about the same time (measured in one process
+# against column order with non-temporal loads: fp16 9999 x 10001 3.52 -> 4.10 TB/s, 16386 x 8191 2.95 -> 3.92,
+# 10000^2 3.78 -> 4.28; fp32 9999 x 10001 3.79 -> 4.48, 8200 x 8192 3.94 -> 4.89; fp16 10000 x 10240 4.72 -> 4.51).
+# What remains is the count of 128-byte lines an access touches: the same kernel on fp16 10048^2 (rows of whole lines)
+# moves 5.3 TB/s, on 10016^2 (whole 64-byte halves) 4.5, on 10000^2 3.8 (a 256-byte row segment touches three lines).
+# fp32 4096^2 (2048 workgroups of 32 KiB, five resident per CU: 1.6 rounds) against tilings whose workgroups make whole
+# rounds: 64x64 tiles in the same windows (4096 workgroups, eight per CU: two rounds) 26.2 us, 32x128 tiles 25.6 us,
+# 64x64 tiles in 32x16 windows 26.8 us, the 64x128 tiles built 24.6 us; a plain copy of the same 2 x 64 MiB takes 22.4 us.
 TRANSPOSE = {
     "f32": [dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 64, 8), max_bytes=1536 << 20),
             dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 32, 8), max_bytes=1536 << 20),
             dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag", min_elements=2 << 20),   # smaller: 64x64 tiles
             dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag"),
-            dict(dtype="f32", tile=(32, 32), group=(2, 4), order="col", edge=True, xcd=True),
-            dict(dtype="f32", tile=(32, 32), group=(4, 2), order="col", edge=True, ragged=True, xcd=True),
+            dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("strip", 8), edge=True, xcd=True),
+            dict(dtype="f32", tile=(32, 32), group=(4, 2), order=("strip", 8), edge=True, ragged=True, xcd=True),
             dict(dtype="f32", tile=(32, 32), group=(2, 2), order="col", edge=True, ragged=True, xcd=True)],
     "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 128, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 64, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 32, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag", min_elements=2 << 20),   # smaller: 64x64 tiles
             dict(dtype="f16", tile=(64, 64), group=(1, 1), order="diag"),
-            dict(dtype="f16", tile=(64, 64), group=(2, 2), order="col", edge=True, xcd=True),
-            dict(dtype="f16", tile=(64, 64), group=(2, 2), order="col", edge=True, ragged=True, xcd=True),
+            dict(dtype="f16", tile=(64, 64), group=(2, 2), order=("strip", 8), edge=True, xcd=True),
+            dict(dtype="f16", tile=(64, 64), group=(2, 2), order=("strip", 8), edge=True, ragged=True, xcd=True),
             dict(dtype="f16", tile=(64, 64), group=(1, 1), order="col", edge=True, ragged=True, xcd=True)],
 }
 # (element type, vectorised, waves per row): 16-byte accesses need N % (16/size) == 0; the
@@ -85,9 +95,11 @@ def collect():
         for cfg in configs:
             cfg = dict(cfg)
             max_bytes = cfg.pop("max_bytes", None)   # only for matrices that fit the last-level cache
+            tuning_only = cfg.pop("tuning_only", False)      # built for comparison, never picked
             min_elements = cfg.pop("min_elements", None)
-            unit, meta = transpose.emit(**cfg, suffix="")
+            unit, meta = transpose.emit(**cfg)
             meta["max_bytes"] = max_bytes
+            meta["tuning_only"] = tuning_only
             if min_elements:
                 meta["min_elements"] = min_elements
             if cfg.get("edge"):
@@ -157,6 +169,8 @@ def collect():
               f"inline hipError_t lego_transpose_{dtype}_dispatch(const void* in, void* out, int rows, int cols, "
               "hipStream_t stream) {"]
         for m in metas:
+            if m["tuning_only"]:
+                continue
             fits = "" if m["max_bytes"] is None else \
                 f" && 2ull * rows * cols * {4 if dtype == 'f32' else 2} <= {m['max_bytes']}ull"
             if m.get("min_side"):
@@ -173,7 +187,15 @@ def collect():
             if m["any_element"]:
                 h.append(f"  if (rows >= {m['min_side']} && cols >= {m['min_side']} && 1ull * rows * cols >= {m['min_elements']}ull) "
                          f"return {m['kernel']}_launch(in, out, rows, cols, stream);")
-        h += [f"  return lego_transpose_any_launch(in, out, rows, cols, {4 if dtype == 'f32' else 2}, stream);", "}", ""]
+        h += [f"  return lego_transpose_any_launch(in, out, rows, cols, {4 if dtype == 'f32' else 2}, stream);", "}",
+              "// tiling number `tiling` of the list above, for a shape it takes (16-byte aligned bases); the caller compares tilings with it",
+              f"inline hipError_t lego_transpose_{dtype}_tiling(int tiling, const void* in, void* out, int rows, int cols, "
+              "hipStream_t stream) {"]
+        for n_, m in enumerate(metas):
+            fits = f" && rows >= {m['min_side']} && cols >= {m['min_side']}" if m.get("min_side") else ""
+            h.append(f"  if (tiling == {n_} && rows % {m['row_multiple']} == 0 && cols % {m['col_multiple']} == 0{fits}) "
+                     f"return {m['kernel']}_launch(in, out, rows, cols, stream);      // {m['SR']} x {m['SC']}")
+        h += ["  return hipErrorInvalidValue;", "}", ""]
     for dtype, vec, w in ROWWISE:
         tag = dtype if vec else dtype + "s"
         h += [f"hipError_t lego_softmax_{tag}_w{w}_launch(const void*, void*, int, int, hipStream_t);",

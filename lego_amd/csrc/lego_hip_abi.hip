@@ -315,6 +315,18 @@ int lego_hip_transpose_f16(const void* in, void* out, int rows, int cols, void* 
   return ok_or(lego_transpose_f16_dispatch(in, out, rows, cols, as_stream(stream)));
 }
 
+int lego_hip_transpose_f32_tiling(const void* in, void* out, int rows, int cols, int tiling, void* stream)
+{
+  if (!aligned16(in) || !aligned16(out) || in == out || rows <= 0 || cols <= 0) return kInvalid;
+  return ok_or(lego_transpose_f32_tiling(tiling, in, out, rows, cols, as_stream(stream)));
+}
+
+int lego_hip_transpose_f16_tiling(const void* in, void* out, int rows, int cols, int tiling, void* stream)
+{
+  if (!aligned16(in) || !aligned16(out) || in == out || rows <= 0 || cols <= 0) return kInvalid;
+  return ok_or(lego_transpose_f16_tiling(tiling, in, out, rows, cols, as_stream(stream)));
+}
+
 int lego_hip_softmax_f16_wpr(const void* x, void* y, int M, int N, int waves_per_row, void* stream)
 {
   if (!usable(x) || !usable(y)) return kInvalid;

@@ -110,7 +110,8 @@ def tile_order(order, n_bi, n_bj, wg):
     that run together spread both their reads and their writes over tile columns -- the
     classic remedy for DRAM channel camping when the row pitch is a power of two;
     ``("window", ti, tj)``: row order inside windows of ``ti x tj`` tiles, windows in row
-    order; ``n_bi`` and ``n_bj`` must be multiples of ``ti`` and ``tj``.
+    order; ``n_bi`` and ``n_bj`` must be multiples of ``ti`` and ``tj``;
+    ``("strip", w)``: row order inside strips of ``w`` tile columns, any ``n_bi`` and ``n_bj``.
     """
     if order == "row":
         return OrderBy(Row(n_bi, n_bj)).TileBy([n_bi, n_bj]).inv(wg)
@@ -129,15 +130,32 @@ def tile_order(order, n_bi, n_bj, wg):
         windows = OrderBy(Row(n_bi / ti, n_bj / tj), Row(ti, tj)).TileBy([n_bi / ti, n_bj / tj], [ti, tj])
         wi, wj, i, j = windows.inv(wg)
         return wi * ti + i, wj * tj + j
+    if isinstance(order, tuple) and order[0] == "strip":
+        # strips of w tile columns (the last one narrower), row order inside a strip: the workgroups in flight cover
+        # a block of tiles some w wide and as many rows deep as fit, so that a tile's neighbours on all four sides
+        # run with it -- for shapes whose tile edges cut 128-byte lines in both matrices
+        _, w = order
+        if isinstance(wg, sp.Expr):
+            strip = sp.Min(sp.floor(wg / (n_bi * w)), sp.floor(n_bj / w))
+            width = sp.Min(w, n_bj - strip * w)
+            rem = wg - strip * n_bi * w
+            return sp.floor(rem / width), strip * w + sp.Mod(rem, width)
+        strip = min(wg // (n_bi * w), n_bj // w)
+        width = min(w, n_bj - strip * w)
+        rem = wg - strip * n_bi * w
+        return rem // width, strip * w + rem % width
     raise ValueError(order)
 
 
-def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix="", edge=False, ragged=False, xcd=False):
+def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix="", edge=False, ragged=False, xcd=False,
+         stream_loads=False):
     """HIP translation unit for one element type and one tiling.  ``edge``: the shape need not be
     a whole number of macro tiles, only of 16-byte vectors in both directions; vectors past the
     edge are skipped.  ``ragged`` (with ``edge``): any shape; rows start at any element, the vectors
     that an edge cuts go element by element.  ``xcd`` (with ``edge``): workgroup ids are dealt to the tiles
-    so that each XCD takes a contiguous run of them (``order`` is then the order inside that run)."""
+    so that each XCD takes a contiguous run of them (``order`` is then the order inside that run).
+    ``stream_loads`` (with ``edge``): non-temporal loads, as the kernels for whole tiles use; without it the 128-byte
+    lines that the row segments of neighbouring tiles share stay in the L2 for the neighbour."""
     elt, esize = {"f32": ("float", 4), "f16": ("_Float16", 2)}[dtype]
     vec = 16 // esize                       # elements per 16-byte vector
     (TR, TC), (MR, MC) = tile, group
@@ -164,7 +182,7 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix="", edge=
 
     # workgroup -> macro tile, row-major over the grid of macro tiles
     nBi, nBj = size("nBi"), size("nBj")
-    windowed = isinstance(order, tuple)
+    windowed = isinstance(order, tuple) and order[0] == "window"
     if windowed:
         # tile counts as multiples of the window, so that every division is exact
         WI, WJ = order[1:]
@@ -207,7 +225,7 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix="", edge=
         grid=(f"(static_cast<unsigned>((rows + {SR - 1}) / {SR}) * static_cast<unsigned>((cols + {SC - 1}) / {SC}) + 7) / 8 * 8" if edge and xcd else
               f"static_cast<unsigned>((rows + {SR - 1}) / {SR}) * static_cast<unsigned>((cols + {SC - 1}) / {SC})" if edge
               else f"static_cast<unsigned>(rows / {SR}) * static_cast<unsigned>(cols / {SC})"),
-        edge=edge, ragged=ragged, VEC=vec, bits_t="uint32_t" if esize == 4 else "uint16_t",
+        edge=edge, ragged=ragged, stream_loads=stream_loads, VEC=vec, bits_t="uint32_t" if esize == 4 else "uint16_t",
         # matrix coordinates of the vectors, for the edge tests: source (row, first column) in phase 1,
         # destination (row = source column, first column = source row) in phase 2
         p1_row=code(tidy(OrderBy(Row(nBi, SR)).TileBy([nBi], [SR])[Bi, r], {r: (0, SR)})),

@@ -20,6 +20,8 @@ SIGNATURES = {
     "lego_hip_abi_version": [],
     "lego_hip_transpose_f32": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "lego_hip_transpose_f16": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+    "lego_hip_transpose_f32_tiling": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    "lego_hip_transpose_f16_tiling": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "lego_hip_softmax_f16": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "lego_hip_softmax_f32": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "lego_hip_softmax_bf16": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
