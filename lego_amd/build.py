@@ -279,10 +279,11 @@ ASM_MFMA_MIN_DISTANCE = 16
 
 
 def asm_mfma_read_distance(assembly: str):
-    """Smallest number of instructions, per function of a gfx950 assembly listing, between an MFMA and the next
+    """Smallest number of issue slots, per function of a gfx950 assembly listing, between an MFMA and the next
     instruction other than an MFMA that names one of the accumulation registers it writes (``a7`` or a range
-    ``a[4:7]``), counted along the listing: ``{function: (distance, register, instruction)}``.  Functions in which
-    no MFMA result is read back are left out."""
+    ``a[4:7]``), counted along the listing: ``{function: (distance, register, instruction)}``.  An instruction
+    counts one slot, an MFMA in between four (it issues no sooner than the matrix core is free of the one before,
+    four passes at least).  Functions in which no MFMA result is read back are left out."""
     import re
     out, name, last, count = {}, None, {}, 0
     for line in assembly.split("\n"):
@@ -293,8 +294,8 @@ def asm_mfma_read_distance(assembly: str):
             continue
         if not text or text[0] in ";." or text.endswith(":"):
             continue
-        count += 1
         m = re.match(r"v_mfma\S+\s+a\[(\d+):(\d+)\]", text)
+        count += 4 if m else 1
         if m:
             for r in range(int(m.group(1)), int(m.group(2)) + 1):
                 last[r] = count

@@ -112,5 +112,6 @@ def test_build_check_finds_an_accumulator_read_close_behind_an_inline_assembly_m
         "\tv_accvgpr_read_b32 v10, a[4:5]\n\ts_endpgm\nkernel_b:\n" + mfma + "\ts_endpgm\n"
     assert build.asm_mfma_read_distance(close) == {"kernel_a": (3, 5, "v_accvgpr_read_b32")}
     found = build.asm_mfma_read_distance(far)
-    assert found == {"kernel_a": (21, 4, "v_accvgpr_read_b32")}      # kernel_b reads nothing back
+    assert found == {"kernel_a": (24, 4, "v_accvgpr_read_b32")}      # an MFMA between counts four; kernel_b reads nothing back
     assert found["kernel_a"][0] >= build.ASM_MFMA_MIN_DISTANCE > 3
+
