@@ -47,16 +47,21 @@ def lds_a_layout(bm, chunks):
     return OrderBy(GenP((bm, chunks), forward, backward)).TileBy([bm, chunks])
 
 
-def lds_b_layout(bk, bn, period=4):
+def lds_b_layout(bk, bn, period=4, groups_by_k=False):
     """B tile in elements, rows of ``bn``: ``k*bn + (n ^ 32*(k % period))``.
 
     A transposing read of 2-byte elements touches four consecutive k-rows, 64 bytes of each;
     rotating the 64-byte chunk index by ``k % 4`` puts the four rows on four different quarters
     of the banks.  One of 1-byte elements touches eight k-rows, 32 bytes of each (32 elements
     again): ``period = 8``.  Bits 0-4 of ``n`` are untouched, so 16-byte stores and 8-byte reads
-    stay whole."""
+    stay whole.  ``groups_by_k`` (16 x 16 MFMA blocks, 2-byte elements): the two 16-lane groups that an 8-byte read
+    serves together read the same 16 columns of k-rows eight apart, 32 of the 64 bytes of each quarter; the key
+    also flips bit 4 of ``n`` (32 bytes) with bit 3 of ``k``, which sends the second group to the other 32 bytes
+    (bits 0-3 stay, so 16-byte stores and 8-byte reads are still whole)."""
+    assert not groups_by_k or period == 4
+
     def key(k):
-        return (k % period) * 32
+        return (k % period) * 32 + (((k // 8) % 2) * 16 if groups_by_k else 0)
 
     def forward(kn):
         k, n = kn
@@ -303,23 +308,30 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
     lrow, lk = (l32, lhi) if block == 32 else (l16, lgrp)
 
     def chunk_walk(expr, n_iters):
-        """``expr`` (a function of the lane ``t`` and the chunk counter ``it``) as
-        ``expr(it=0) + it*step`` with a lane-independent ``step``; raises if it is not."""
+        """``expr`` (a function of the lane ``t`` and the chunk counter ``it``) as ``base[it % 2] + it*step`` with a
+        lane-independent ``step``: ``(base[0], base[1], step)``, the two bases equal when the walk is affine (they
+        differ where the LDS layout's key changes with the parity of the instruction); raises if it is neither."""
         lane_s, rng_l = idx("lane"), {idx("lane"): (0, 64), wave: (0, WAVES_M * WAVES_N)}
         at = [tidy(sp.sympify(expr).subs(it, v), rng_l) for v in range(n_iters)]
-        step = sp.simplify(at[1] - at[0]) if n_iters > 1 else sp.Integer(0)
-        if step.free_symbols & {lane_s, wave}:
+        two = sp.simplify(at[2] - at[0]) if n_iters > 2 else sp.simplify(2 * (at[1] - at[0])) if n_iters > 1 else sp.Integer(0)
+        if two.free_symbols & {lane_s, wave}:
             # not visibly uniform: decide by exhaustive evaluation below
-            step = sp.simplify((at[1] - at[0]).subs({lane_s: 0, wave: 0}))
-        sizes = {s_: 8192 + 256 * n_ for n_, s_ in enumerate(sorted(step.free_symbols | at[0].free_symbols
-                                                                   - {lane_s, wave}, key=str))}
-        for v in range(n_iters):   # exhaustive over lanes and waves: the walk really is affine
-            diff = sp.lambdify([lane_s, wave], (at[v] - at[0] - v * step).subs(sizes), "math")
+            two = sp.simplify(two.subs({lane_s: 0, wave: 0}))
+        step = sp.simplify(two / 2)
+        base = [at[0], tidy(at[1] - step, rng_l) if n_iters > 1 else at[0]]
+        names = sorted(set().union(*(e.free_symbols for e in at + [step])) - {lane_s, wave}, key=str)
+        sizes = {s_: 8192 + 256 * n_ for n_, s_ in enumerate(names)}
+        evaluate = [{"BitXor": lambda a_, b_: int(a_) ^ int(b_)}, "math"]
+        same = True
+        for v in range(n_iters):   # exhaustive over lanes and waves
+            diff = sp.lambdify([lane_s, wave], (at[v] - base[v % 2] - v * step).subs(sizes), evaluate)
+            gap = sp.lambdify([lane_s, wave], (base[1] - base[0]).subs(sizes), evaluate)
             for w_ in range(WAVES_M * WAVES_N):
                 for l_ in range(64):
                     if diff(l_, w_) != 0:
-                        raise ValueError("chunk offsets are not affine in the instruction counter")
-        return at[0], step
+                        raise ValueError("chunk offsets are not affine in the instruction counter, by parity either")
+                    same = same and gap(l_, w_) == 0
+        return base[0], (base[0] if same else base[1]), step
 
     Cs_L = lds_c_layout(WM, WN, block)
     cp = idx("cp")
@@ -394,7 +406,7 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
             else:
                 frag = "read_k_fragment(%s)" % ", ".join("%ss + (%s)" % (role, c) for c in chunks)
         else:
-            lds = lds_b_layout(bk, rows, 4 if esize == 2 else 8)
+            lds = lds_b_layout(bk, rows, 4 if esize == 2 else 8, groups_by_k=block == 16)
             kr_e, col_e = (tidy(e, slot_rng) for e in lds.inv(EPC * slot))
             full = tidy(glob(EPC * ch, kr), rng)    # here `ch` counts 16-byte chunks along the row
             placed = full.subs({kr: kr_e, ch: tidy(col_e / EPC, slot_rng)})
@@ -414,15 +426,19 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
                 frag_c = wave_off + (lgrp % 2) * 16 + 8 * (l16 % 2)
             frag = ("read_t_fragment(%s)"
                     % ", ".join("%ss + (%s)" % (role, code(tidy(lds[fk, frag_c], rng))) for fk in frag_k))
-        src0, step = chunk_walk(placed.subs({tile_id: 0, k: 0}), n_iters)
+        src0, src1, step = chunk_walk(placed.subs({tile_id: 0, k: 0}), n_iters)
         # what bounds a chunk at a ragged edge: its row of the tile (k-major: the row changes with the
-        # instruction) or its first column (the other kind: the same for every instruction)
-        edge0, edge_step = chunk_walk(r_e if kmajor else col_e, n_iters)
+        # instruction) or its first column (the other kind: the same for every instruction, or one of two by
+        # the instruction's parity)
+        edge0, edge1, edge_step = chunk_walk(r_e if kmajor else col_e, n_iters)
         assert kmajor or edge_step == 0
         # the first k-value (within the tile) of a lane's chunk: what a ragged last k-tile is masked by
-        kedge0, kedge_step = chunk_walk(EPC * ch_e if kmajor else kr_e, n_iters)
+        kedge0, kedge1, kedge_step = chunk_walk(EPC * ch_e if kmajor else kr_e, n_iters)
+        assert kedge1 is kedge0
         return {f"{role}_src0": code(src0), f"{role}_src_step": code(step),
+                f"{role}_src0_odd": None if src1 is src0 else code(src1),
                 f"{role}_edge0": code(edge0), f"{role}_edge_step": code(edge_step),
+                f"{role}_edge0_odd": None if edge1 is edge0 else code(edge1),
                 f"{role}_kedge0": code(kedge0), f"{role}_kedge_step": code(kedge_step),
                 f"{role}_goff_base": code(full.subs({k: 0, row: 0, ch: 0, kr: 0})),
                 f"{role}_kstep": code(sp.simplify(full.subs(k, k + 1) - full)),

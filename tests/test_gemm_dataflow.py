@@ -64,14 +64,17 @@ def test_fragments_receive_the_right_elements(dtype, bk, tile, block, variant):
     for role, rows_total, kmajor in (("a", M, not ta), ("b", N, tb)):
         src0 = _grab(text, r"const unsigned %s_src0 = \d \* \((.*)\);" % role)
         step = _grab(text, r"%s_src_step = \d \* \((.*?)\)[,;]" % role)
+        # (the lane's offset for odd instructions, where the LDS layout's key changes with the instruction's parity)
+        odd = re.search(r"const unsigned %s_src0_odd = \d \* \((.*)\);" % role, text)
+        src0_odd = odd.group(1) if odd else src0
         iters = tile * bk // epc // 256
         # --- what the memory->LDS instructions leave in the LDS buffer: element ids of tile (0, 0)
         lds = np.full(tile * bk, -1, dtype=np.int64)
         for wave in range(4):
             for lane in range(64):
-                base = _c_eval(src0, dict(sizes, wave=wave, lane=lane))
+                bases = [_c_eval(e, dict(sizes, wave=wave, lane=lane)) for e in (src0, src0_odd)]
                 for it in range(iters):
-                    off = base + it * _c_eval(step, sizes)          # element offset inside the operand
+                    off = bases[it % 2] + it * _c_eval(step, sizes)          # element offset inside the operand
                     slot = (it * 4 + wave) * 64 + lane
                     # element id = (row, k) of the tile: k-major storage has pitch K, the other pitch rows_total
                     for e in range(epc):
@@ -124,35 +127,42 @@ def test_fragments_receive_the_right_elements(dtype, bk, tile, block, variant):
                         assert got[lane].tolist() == [row * bk + k0 + x for x in range(kk)], (role, ks, sub, w, lane)
 
 
-@pytest.mark.parametrize("tile", [256, 128])
+@pytest.mark.parametrize("tile,block", [(256, 32), (256, 16), (128, 32)])
 @pytest.mark.parametrize("variant", ["nn", "nt", "tn", "tt"])
-def test_ragged_edges_skip_exactly_what_lies_outside(variant, tile):
+def test_ragged_edges_skip_exactly_what_lies_outside(variant, tile, block):
     """The EDGE instantiation runs memory->LDS instruction ``x`` under the mask of the lanes with
     ``edge0 + x*step < rem``.  For a tile with ``rem`` valid rows (columns), replay the masks: every chunk that
     passes must lie inside the operand, and every chunk with data of a valid row (column) must pass."""
     ta, tb = variant[0] == "t", variant[1] == "t"
     bk = 64
-    unit, _ = gemm.emit(bm=tile, bn=tile, bk=bk, trans_a=ta, trans_b=tb, with_grouped=False)
+    unit, _ = gemm.emit(bm=tile, bn=tile, bk=bk, trans_a=ta, trans_b=tb, with_grouped=False, block=block)
     text = unit.text
     K = 2 * bk
+    edge_odds = re.search(r"const unsigned a_edge0_odd = (.*), b_edge0_odd = (.*);", text).groups()
     for role, kmajor in (("a", not ta), ("b", tb)):
         src0 = _grab(text, r"const unsigned %s_src0 = \d \* \((.*)\);" % role)
         step = _grab(text, r"%s_src_step = \d \* \((.*?)\)[,;]" % role)
+        # (the lane's offset for odd instructions, where the LDS layout's key changes with the instruction's parity)
+        odd = re.search(r"const unsigned %s_src0_odd = \d \* \((.*)\);" % role, text)
+        src0_odd = odd.group(1) if odd else src0
         edge0 = _grab(text, r"const unsigned a_edge0 = (.*), b_edge0 = .*;") if role == "a" else \
             _grab(text, r"const unsigned a_edge0 = .*, b_edge0 = (.*);")
-        estep = int(_grab(text, r"%s_edge0 \+ x \* \((\d+)\) < %s_rem" % (role, "m" if role == "a" else "n")))
+        edge0_odd = edge_odds[role == "b"]
+        if edge0_odd == role + "_edge0":
+            edge0_odd = edge0
+        estep = int(_grab(text, r"%s_edge0\) \+ x \* \((\d+)\) < %s_rem" % (role, "m" if role == "a" else "n")))
         for rem in (r for r in (8, 40, 120, 128, 200, 248) if r <= tile):
             rows_total = rem                     # the operand ends where the tile's valid part ends
             sizes = dict(M=rows_total, N=rows_total, K=K)
             covered = set()
             for wave in range(4):
                 for lane in range(64):
-                    base = _c_eval(src0, dict(sizes, wave=wave, lane=lane))
-                    e0 = _c_eval(edge0, dict(wave=wave, lane=lane))
+                    bases = [_c_eval(e, dict(sizes, wave=wave, lane=lane)) for e in (src0, src0_odd)]
+                    e0s = [_c_eval(e, dict(wave=wave, lane=lane)) for e in (edge0, edge0_odd)]
                     for it in range(tile * bk // 8 // 256):
-                        if not e0 + it * estep < rem:
+                        if not e0s[it % 2] + it * estep < rem:
                             continue
-                        off = base + it * _c_eval(step, sizes)
+                        off = bases[it % 2] + it * _c_eval(step, sizes)
                         # the chunk's eight elements must exist: pitch K (k-major) or rows_total
                         for e in range(8):
                             if kmajor:
@@ -164,9 +174,9 @@ def test_ragged_edges_skip_exactly_what_lies_outside(variant, tile):
             assert covered == {(r, k) for r in range(rem) for k in range(bk)}, (role, rem)
 
 
-@pytest.mark.parametrize("dtype,bk", [("f16", 64), ("e5m2", 128)])
+@pytest.mark.parametrize("dtype,bk,block", [("f16", 64, 32), ("f16", 64, 16), ("e5m2", 128, 32)])
 @pytest.mark.parametrize("variant", ["nn", "tt"])
-def test_last_k_tile_zeroes_exactly_what_lies_past_k(dtype, bk, variant):
+def test_last_k_tile_zeroes_exactly_what_lies_past_k(dtype, bk, block, variant):
     """In the last k-tile of a ragged K the EDGE instantiation keeps a lane in instruction ``x``'s mask while
     ``k0 + x*step < klim``: the slots of the other lanes are written as zeros, once, instead of being fetched.
     For every ``klim`` in whole chunks, replay the guards
@@ -175,7 +185,7 @@ def test_last_k_tile_zeroes_exactly_what_lies_past_k(dtype, bk, variant):
     ``klim`` and zeros above."""
     ta, tb = variant[0] == "t", variant[1] == "t"
     tile = 256
-    unit, _ = gemm.emit(bm=tile, bn=tile, bk=bk, trans_a=ta, trans_b=tb, with_grouped=False, dtype=dtype)
+    unit, _ = gemm.emit(bm=tile, bn=tile, bk=bk, trans_a=ta, trans_b=tb, with_grouped=False, dtype=dtype, block=block)
     text = unit.text
     esize = 2 if dtype == "f16" else 1
     epc = 16 // esize
@@ -185,16 +195,19 @@ def test_last_k_tile_zeroes_exactly_what_lies_past_k(dtype, bk, variant):
     for role, rows_total, kmajor, k0_text in (("a", 512, not ta, k0s[0]), ("b", 512, tb, k0s[1])):
         src0 = _grab(text, r"const unsigned %s_src0 = \d \* \((.*)\);" % role)
         step = _grab(text, r"%s_src_step = \d \* \((.*?)\)[,;]" % role)
+        # (the lane's offset for odd instructions, where the LDS layout's key changes with the instruction's parity)
+        odd = re.search(r"const unsigned %s_src0_odd = \d \* \((.*)\);" % role, text)
+        src0_odd = odd.group(1) if odd else src0
         kstep = int(_grab(text, r"%s_k0 \+ x \* \((\d+)\) < klim_nx" % role))
         iters = tile * bk // epc // 256
         for klim in range(epc, bk + 1, epc):
             zeroed, fetched = set(), set()
             for wave in range(4):
                 for lane in range(64):
-                    base = _c_eval(src0, dict(sizes, wave=wave, lane=lane))
+                    bases = [_c_eval(e, dict(sizes, wave=wave, lane=lane)) for e in (src0, src0_odd)]
                     k0 = _c_eval(k0_text, dict(wave=wave, lane=lane))
                     for it in range(iters):
-                        off = base + it * _c_eval(step, sizes)
+                        off = bases[it % 2] + it * _c_eval(step, sizes)
                         r_, k_ = divmod(off, K) if kmajor else divmod(off, rows_total)[::-1]
                         assert k_ == k0 + it * kstep, (role, wave, lane, it)      # the guard sees the chunk's own k
                         (zeroed if k0 + it * kstep >= klim else fetched).add((r_, k_))

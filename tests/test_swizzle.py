@@ -101,6 +101,27 @@ def test_gemm_lds_layouts_are_bijective_and_conflict_free():
             assert conflicts(addrs, 2) == 1
 
 
+def test_gemm_lds_layout_for_16_column_blocks_is_bijective_and_conflict_free():
+    """v_mfma_f32_16x16x32: a fragment's four lane groups are four k blocks of the same 16 columns, so the two groups
+    of a pass read the same columns of k-rows eight apart; the layout's key tells them apart (without it the test
+    below counts two addresses per bank, and the GEMM measures SQ_LDS_BANK_CONFLICT at a third of its LDS cycles)."""
+    bn, bk = 256, 64
+    b = gemm.lds_b_layout(bk, bn, 4, groups_by_k=True)
+    tb = np.array([[int(b.apply(k, n)) for n in range(bn)] for k in range(bk)])
+    assert sorted(tb.ravel().tolist()) == list(range(bk * bn))
+    for wave in range(4):      # global->LDS: chunk (t % 32) of k-row (t / 32)
+        lanes = [wave * 64 + l for l in range(64)]
+        assert conflicts([tb[t // 32, 8 * (t % 32)] // 2 for t in lanes], 4, write=True) == 1
+    plain = gemm.lds_b_layout(bk, bn, 4)
+    tp = np.array([[int(plain.apply(k, n)) for n in range(bn)] for k in range(bk)])
+    for ks in range(2):
+        for h in range(2):
+            for j in range(16):
+                rows_cols = [(ks * 32 + (l // 16) * 8 + h * 4 + (l % 16) // 4, 16 * j + 4 * (l % 4)) for l in range(64)]
+                assert conflicts([tb[k, n] // 2 for k, n in rows_cols], 2) == 1
+                assert conflicts([tp[k, n] // 2 for k, n in rows_cols], 2) == 2
+
+
 def test_gemm_lds_layouts_8bit_are_bijective_and_conflict_free():
     """One-byte operands: 128 k-values per tile, 32 per lane and MFMA."""
     bm, bn, bk = 256, 256, 128
