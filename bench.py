@@ -64,10 +64,11 @@ def main():
     ap.add_argument("--sustain", type=float, default=0.0, metavar="SECONDS",
                     help="after timing the 8192^3 GEMM, keep launching it back to back for this long (for sampling "
                          "socket power and clocks with amd-smi from another process) and report the sustained rate")
-    ap.add_argument("--only", default="", help="comma list of configs to time (c1,c2,c3,c4,c5,extra,apps,energy); "
+    ap.add_argument("--only", default="", help="comma list of configs to time (c1,c2,c3,c4,c5,extra,apps,energy,timeline); "
                     "c2 is always timed; 'extra' adds LayerNorm backward and the other GEMM layouts and element "
                     "types, 'apps' the stencil, Needleman-Wunsch and LUD programs, 'energy' (with c4) the sustained "
-                    "comparison of GEMM variants and MFMA-only streams for power sampling")
+                    "comparison of GEMM variants and MFMA-only streams for power sampling, 'timeline' (when named) the "
+                    "per-phase times of the tiles of the fp16 GEMM and grouped GEMM from their measurement build")
     ns = ap.parse_args()
     if ns.gpus != 1:
         print("bench.py: this build measures one MI355X; every configuration of the hot path is a "
@@ -567,6 +568,28 @@ def main():
         plan5 = (ctypes.c_int * 3)()
         runtime.call("lego_hip_grouped_gemm_f16_plan", sz, 8, plan5)
         kernels["c5_grouped_gemm_f16"]["launch"] = dict(tile=plan5[0], tiles=plan5[1], tiles_split_in_halves=plan5[2])
+        if ns.sustain > 0:
+            # The grouped launch back to back for --sustain seconds, then one GEMM of four exactly full rounds of the same
+            # 16-k-tile tiles (8192 x 8192 x 1024), with wall-clock times for power and clock samples taken by another process.
+            a1k = (torch.randn(8192, 1024, generator=g5) / 32).half().to(dev)
+            b1k = (torch.randn(1024, 8192, generator=g5) / 32).half().to(dev)
+            c1k = torch.empty(8192, 8192, dtype=torch.half, device=dev)
+            table = []
+            for label, flop, fn in (("grouped GEMM, config 5", fl5, gg),
+                                    ("gemm 8192 x 8192 x 1024 (1024 tiles of 16 k-tiles: four full rounds)", 2.0 * 8192 * 8192 * 1024,
+                                     lambda: runtime.call("lego_hip_gemm_f16", p(a1k), p(b1k), p(c1k), 8192, 8192, 1024, stream))):
+                per = []
+                t_begin = time.time()
+                t_end = time.perf_counter() + ns.sustain
+                while time.perf_counter() < t_end:
+                    per.append(timed(fn, steps=200, warmup=1, settle_ms=0.0))
+                steady = per[len(per) // 3:]
+                table.append(dict(variant=label, tflops=flop / (sum(steady) / len(steady)) / 1e9, wall_clock_begin=t_begin,
+                                  wall_clock_end=time.time()))
+                print(f"{t_begin:.2f} .. {time.time():.2f}  {label}: {table[-1]['tflops']:.1f} TFLOP/s", file=sys.stderr, flush=True)
+                time.sleep(1.0)
+            kernels["c5_sustained"] = table
+            del a1k, b1k, c1k
         if not ns.skip_cpu:
             from oracle import kernels as ok5
             Ac, Bc = [t.cpu() for t in A], [t.cpu() for t in B]
@@ -575,6 +598,73 @@ def main():
                 "all 8 problems: (A.float() @ B.float()).half() each")
             del Ac, Bc
         del A, B, C
+
+    # ---- where the time of a GEMM tile goes: the measurement build of the fp16 kernels (same tiles and schedules) ------
+    if "timeline" in only:
+        import numpy as np
+        g5 = gen(5)
+        idx = torch.randint(0, 3, (8, 3), generator=g5)
+        dims = [[(1024, 2048, 4096)[int(v)] for v in row] for row in idx]
+        A = [(torch.randn(m, k, generator=g5) / math.sqrt(k)).half().to(dev) for m, n, k in dims]
+        B = [(torch.randn(k, n, generator=g5) / math.sqrt(k)).half().to(dev) for m, n, k in dims]
+        C = [torch.empty(m, n, dtype=torch.half, device=dev) for m, n, k in dims]
+        arr = ctypes.c_void_p * 8
+        pa, pb, pc = arr(*[t.data_ptr() for t in A]), arr(*[t.data_ptr() for t in B]), arr(*[t.data_ptr() for t in C])
+        sz = (ctypes.c_int * 24)(*[v for d in dims for v in d])
+        plan5 = (ctypes.c_int * 3)()
+        runtime.call("lego_hip_grouped_gemm_f16_plan", sz, 8, plan5)
+        at = (torch.randn(8192, 8192, generator=g5) / 90.5).half().to(dev)
+        bt = (torch.randn(8192, 8192, generator=g5) / 90.5).half().to(dev)
+        ct = torch.empty(8192, 8192, dtype=torch.half, device=dev)
+
+        def plain(k):
+            return lambda: runtime.call("lego_hip_gemm_f16_variant", p(at), p(bt), p(ct), 8192, 8192, k, 3, stream)
+        runtime.call("lego_hip_grouped_gemm_f16_stamps", pa, pb, pc, sz, 8, stream)
+        torch.cuda.synchronize()
+        assert max(((c.float() - a.float() @ b.float()).norm() / (a.float() @ b.float()).norm()).item()
+                   for a, b, c in zip(A, B, C)) <= 1e-2
+        names = ("entry -> first k-tile in LDS", "-> first fragments read", "main loop and the k-tile before the last",
+                 "slots of the last k-tile (results leave under them)", "tail: last staging and stores issued",
+                 "last stores leave")
+        table = []
+        for label, wgs, flop, fn in (
+                ("grouped GEMM, config 5", plan5[1] + plan5[2], sum(2.0 * m * n * k for m, n, k in dims),
+                 lambda: runtime.call("lego_hip_grouped_gemm_f16_stamps", pa, pb, pc, sz, 8, stream)),
+                ("gemm 8192 x 8192 x 1024", 1024, 2.0 * 8192 * 8192 * 1024, plain(1024)),
+                ("gemm 8192 x 8192 x 8192", 1024, 2.0 * 8192 ** 3, plain(8192))):
+            ms_t = timed(fn, steps=20, warmup=3)          # the stamps of the last launch of a steady run stay
+            rows = np.zeros(8 * wgs, dtype=np.uint64)
+            runtime.call("lego_hip_gemm_stamps_read", rows.ctypes.data_as(ctypes.c_void_p), wgs)
+            st = rows.reshape(wgs, 8)
+            tus = (st[:, :7].astype(np.int64) - int(st[:, 0].min())) * 0.01          # 100 MHz counter -> microseconds
+            where = ((st[:, 7] >> np.uint64(8)) & np.uint64(0xff)) | ((st[:, 7] >> np.uint64(16)) << np.uint64(8))
+            span = float(tus[:, 6].max())
+            phases = {nm: dict(mean=float(d.mean()), p10=float(np.percentile(d, 10)), p90=float(np.percentile(d, 90)))
+                      for nm, d in zip(names, (tus[:, i + 1] - tus[:, i] for i in range(6)))}
+            busy, gaps, first, last_idle = [], [], [], []
+            for cu in np.unique(where):
+                own = tus[where == cu]
+                own = own[np.argsort(own[:, 0])]
+                busy.append(float((own[:, 6] - own[:, 0]).sum()))
+                first.append(float(own[0, 0]))
+                last_idle.append(span - float(own[-1, 6]))
+                gaps += [float(own[i + 1, 0] - own[i, 6]) for i in range(len(own) - 1)]
+            entry = dict(workload=label, workgroups=wgs, ms=ms_t, tflops=flop / ms_t / 1e9, span_us=span,
+                         workgroup_us_mean=float((tus[:, 6] - tus[:, 0]).mean()), phases_us=phases,
+                         cus_seen=int(len(busy)), cu_busy_fraction=float(np.mean(busy)) / span,
+                         cu_first_start_us_mean=float(np.mean(first)), cu_idle_after_last_us_mean=float(np.mean(last_idle)),
+                         gap_between_workgroups_on_a_cu_us=dict(mean=float(np.mean(gaps)) if gaps else 0.0,
+                                                                p90=float(np.percentile(gaps, 90)) if gaps else 0.0,
+                                                                per_cu_total_mean=float(np.sum(gaps)) / len(busy)),
+                         start_us_deciles=[float(v) for v in np.percentile(tus[:, 0], range(0, 101, 10))],
+                         end_us_deciles=[float(v) for v in np.percentile(tus[:, 6], range(0, 101, 10))])
+            table.append(entry)
+        kernels["gemm_tile_timeline"] = dict(
+            note="measurement build (lane 0 of each workgroup stores the 100 MHz real-time counter at seven points and "
+                 "the CU it ran on); last launch of 20 back-to-back ones after the settle phase; cu_busy_fraction = "
+                 "time between a workgroup's entry and its last store leaving, summed per CU, over the kernel's span",
+            workloads=table)
+        del A, B, C, at, bt, ct
 
     # ---- next rows: the reference's lego_c benchmark programs (stencils on bricks, Needleman-Wunsch, LUD) ----
     if want("apps"):

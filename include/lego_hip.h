@@ -244,8 +244,24 @@ int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const 
  * with the kernel chosen by the caller: variant 0 = what lego_hip_gemm_f16 launches for large products (four waves of
  * 128 x 128, one per SIMD with 256 accumulator registers, v_mfma_f32_16x16x32_f16), 1 = the same workgroup with
  * v_mfma_f32_32x32x16_f16, 2 = eight waves of 128 x 64, two per SIMD with 128 accumulator registers each
- * (v_mfma_f32_32x32x16_f16).  Used by the benchmark to compare them.  No counterpart in the reference. */
+ * (v_mfma_f32_32x32x16_f16), 3 = the measurement build of variant 0 (below).  Used by the benchmark to compare
+ * them.  No counterpart in the reference. */
 int lego_hip_gemm_f16_variant(const void* a, const void* b, void* c, int M, int N, int K, int variant, void* stream);
+
+/* Measurement aid (no counterpart in the reference): where the time of a tile goes.  A second build of the fp16
+ * 256 x 256-tile kernels, plain and grouped, same tiles and instruction schedules, in which lane 0 of every
+ * workgroup with an id below 8192 stores the 100 MHz real-time counter at seven points of its tile and, once,
+ * where it ran.  lego_hip_gemm_f16_variant(..., 3, ...) launches the plain kernel,
+ * lego_hip_grouped_gemm_f16_stamps the grouped one with the launch that lego_hip_grouped_gemm_f16 would choose
+ * (at most 64 problems in whole tiles; a problem set that the entry point would give to the 128 x 128 tiles is refused).
+ * lego_hip_gemm_stamps_read copies the rows of the first `workgroups` workgroup ids of the last such launch to the
+ * host (eight 64-bit words each; it synchronises with the device): words 0..6 = entry, first k-tile in LDS, first
+ * fragments read, main loop and the k-tile before the last done, the last k-tile's slots issued, the last stores
+ * issued, the stores gone; word 7 = the hardware id of the wave (bits 0-15: HW_ID with SIMD, CU, shader array and
+ * engine) and the XCD (bits 16-19).  bench.py --only timeline prints the per-phase table. */
+int lego_hip_grouped_gemm_f16_stamps(const void* const* a, const void* const* b, void* const* c,
+                                     const int* sizes3, int groups, void* stream);
+int lego_hip_gemm_stamps_read(unsigned long long* host, int workgroups);
 
 /* Measurement aid: out[0..bytes) = in[0..bytes), 16 bytes per lane per access, bytes % 16 == 0.
  * No counterpart in the reference.  bench.py uses it as the same-run copy ceiling and the

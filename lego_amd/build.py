@@ -149,7 +149,12 @@ def collect():
     # waits).  8192^3: 1.29 and 1.28 PFLOP/s against 1.36.
     g32, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK["f16"]), dtype="f16", with_grouped=False, suffix="_m32")
     g8, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK["f16"], waves=GEMM_WAVES_TWO_PER_SIMD), dtype="f16", with_grouped=False)
-    units += [g32, g8]
+    # A measurement build of the fp16 kernels as launched (same tiles, same schedules): lane 0 of every workgroup
+    # records the real-time counter at seven points of its tile and the CU it ran on, for the per-phase tables of
+    # bench.py --only timeline.
+    gst, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK["f16"]), dtype="f16", block=GEMM_MFMA_BLOCK["f16"], with_grouped=True,
+                       with_split=True, suffix="_stamps", stamps=True)
+    units += [g32, g8, gst]
     units.append(gemm.emit_any())
     lbs, mlb = layernorm_bwd.emit()
     units += lbs
@@ -243,6 +248,12 @@ def collect():
           "const void* const*, void* const*, const int*, int, hipStream_t);",
           "hipError_t lego_gemm_f16_nn_w2x4_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);",
           "hipError_t lego_gemm_f16_nn_m32_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);",
+          "hipError_t lego_gemm_f16_nn_stamps_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);",
+          "hipError_t lego_grouped_gemm_f16_stamps_launch(const void* const*, const void* const*, void* const*, "
+          "const int*, int, hipStream_t);",
+          "hipError_t lego_grouped_gemm_f16_stamps_split_launch(const void* const*, const void* const*, void* const*, "
+          "const int*, int, int, hipStream_t);",
+          "hipError_t lego_gemm_stamps_read(unsigned long long*, int);",
           "hipError_t lego_gemm_any_launch(const void*, const void*, void*, int, int, int, int, int, int, int, hipStream_t);",
           "hipError_t lego_grouped_gemm_f16_split_launch(const void* const*, const void* const*, void* const*, "
           "const int*, int, int, hipStream_t);",

@@ -756,6 +756,7 @@ int lego_hip_gemm_f16_variant(const void* a, const void* b, void* c, int M, int 
   if (variant == 0) return ok_or(lego_gemm_f16_nn_launch(a, b, c, M, N, K, 0, as_stream(stream)));
   if (variant == 1) return ok_or(lego_gemm_f16_nn_m32_launch(a, b, c, M, N, K, 0, as_stream(stream)));
   if (variant == 2) return ok_or(lego_gemm_f16_nn_w2x4_launch(a, b, c, M, N, K, 0, as_stream(stream)));
+  if (variant == 3) return ok_or(lego_gemm_f16_nn_stamps_launch(a, b, c, M, N, K, 0, as_stream(stream)));
   return kInvalid;
 }
 
@@ -1048,6 +1049,22 @@ int lego_hip_grouped_gemm_f16_split(const void* const* a, const void* const* b, 
   if (split_tiles < 0)
     return ok_or(lego_grouped_gemm_f16_t128x128_launch(a, b, c, sizes3, groups, as_stream(stream)));
   return ok_or(lego_grouped_gemm_f16_split_launch(a, b, c, sizes3, groups, split_tiles, as_stream(stream)));
+}
+
+int lego_hip_grouped_gemm_f16_stamps(const void* const* a, const void* const* b, void* const* c,
+                                     const int* sizes3, int groups, void* stream)
+{
+  if (groups > LEGO_GROUPED_MAX_GROUPS || grouped_check(a, b, c, sizes3, groups) != 0) return kInvalid;
+  const GroupedPlan plan = grouped_plan(sizes3, groups);
+  if (plan.kind == 1) return kInvalid;        // the measurement build exists for the 256 x 256 tiles only
+  if (plan.split == 0) return ok_or(lego_grouped_gemm_f16_stamps_launch(a, b, c, sizes3, groups, as_stream(stream)));
+  return ok_or(lego_grouped_gemm_f16_stamps_split_launch(a, b, c, sizes3, groups, plan.split, as_stream(stream)));
+}
+
+int lego_hip_gemm_stamps_read(unsigned long long* host, int workgroups)
+{
+  if (host == nullptr) return kInvalid;
+  return ok_or(lego_gemm_stamps_read(host, workgroups));
 }
 
 int lego_hip_copy16(const void* in, void* out, unsigned long long bytes, void* stream)

@@ -23,6 +23,7 @@ from .common import BANNER, Emitted, code, idx, size, template, tidy
 XCDS = 8
 CUS = 256      # MI355X: 8 XCDs of 32 CUs
 MAX_GROUPS = 64
+STAMP_ROWS = 8192      # workgroups whose time stamps a measurement build keeps
 
 
 def lds_a_layout(bm, chunks):
@@ -224,7 +225,7 @@ def last_ktile_schedule(TM, TN, NPH, WN, block=32, mps=1):
     return slots, tail
 
 
-def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped, dtype, block=32, suffix=""):
+def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped, dtype, block=32, suffix="", stamps=False):
     """Everything the templates need for one tile shape.  ``block``: 32 = v_mfma_f32_32x32x16 (x64 for 8-bit operands),
     16 = v_mfma_f32_16x16x32 (16-bit operands), the side of an accumulator block."""
     # element type, bytes per element, k-depth of one MFMA, result type; the 8-bit types are the
@@ -470,7 +471,7 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
         # pair together and (32 x 32 blocks) swaps its halves on odd rows
         c_out_row=code(c_out[0]), c_out_pair=code(c_out[1]),
         c_stage_load=code(tidy(4 * Cs_L[cr, 2 * cp], rng) - (4 * (cr % 2) if block == 32 else 0)),
-        BLOCK=block, MPS=MPS, ACC_REGS=block * block // 64, SWAP_ODD_ROWS=block == 32,
+        BLOCK=block, MPS=MPS, ACC_REGS=block * block // 64, SWAP_ODD_ROWS=block == 32, STAMPS=stamps, STAMP_ROWS=STAMP_ROWS,
         c_goff=code(tidy(C_L[pid_m, pid_n, wm * WM + cr, wn * WN + 8 * cp], rng)),
         c_stage_lane=code(stage_lane), c_back_lane=code(back_lane),
         c_wave=code(c_wave_e), c_lane=code(c_lane_e), c_it_step=code(c_it_e),
@@ -503,21 +504,22 @@ def split_order(split, wg):
 
 
 def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, trans_b=False, with_grouped=True,
-         dtype="f16", with_split=False, with_splitk=False, block=32, suffix=""):
+         dtype="f16", with_split=False, with_splitk=False, block=32, suffix="", stamps=False):
     """One translation unit: the GEMM kernel of one operand layout and element type on ``bm x bn``
     tiles, with ``with_grouped`` the grouped kernel on the same tiles, and with ``with_split`` a
     second grouped kernel that gives the last tiles of its launch to two workgroups each, as
     halves of ``bm/2 x bn`` (the tail of a launch whose last round of whole tiles would leave most
     CUs idle).  ``block``: the side of the MFMA's accumulator block (see ``_tile_params``); ``suffix`` goes behind
-    the names of the file and the launchers (a second build of one shape)."""
+    the names of the file and the launchers (a second build of one shape); ``stamps``: a measurement build whose
+    workgroups record the real-time counter at fixed points of their tile (``lego_gemm_stamps_read``)."""
     assert not (with_splitk and block != 32), "partial sums along K are laid out for 32 x 32 accumulator blocks"
-    params = _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped, dtype, block, suffix)
+    params = _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped, dtype, block, suffix, stamps)
     ns = f"t{bm}x{bn}"
     tiles = [dict(ns=ns, text=template("gemm_tile.hip.j2").render(**params))]
     params.update(main_ns=ns, with_split=with_split, with_splitk=with_splitk)
     if with_split:
         assert with_grouped
-        half = _tile_params(bm // 2, bn, bk, waves, max_group_m, trans_a, trans_b, True, dtype, block)
+        half = _tile_params(bm // 2, bn, bk, waves, max_group_m, trans_a, trans_b, True, dtype, block, stamps=stamps)
         hns = f"t{bm // 2}x{bn}"
         tiles.append(dict(ns=hns, text=template("gemm_tile.hip.j2").render(**half)))
         split, swg, ti, hf = size("split"), idx("swg"), idx("pid_m"), idx("half")
@@ -537,6 +539,8 @@ def emit(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8, trans_a=False, tran
         launchers.append(f"lego_grouped_gemm_f16{tag}_split_launch")
     if with_splitk:
         launchers.append(f"lego_gemm_{dtype}_{variant}{tag}_splitk_launch")
+    if stamps:
+        launchers.append("lego_gemm_stamps_read")
     return Emitted(f"gemm_{dtype}_{variant}{tag}.hip", text, launchers), meta
 
 
