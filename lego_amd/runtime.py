@@ -67,6 +67,8 @@ SIGNATURES = {
     "lego_hip_copy16_stream": [_c_void_p, _c_void_p, ctypes.c_ulonglong, _c_void_p],
     "lego_hip_hbm_probe": [_c_void_p, _c_void_p, ctypes.c_ulonglong, _c_int, _c_int, _c_void_p],
     "lego_hip_mfma_probe": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    "lego_hip_grouped_gemm_f16_stamps": [_PTR_ARRAY, _PTR_ARRAY, _PTR_ARRAY, _INT_ARRAY, _c_int, _c_void_p],
+    "lego_hip_gemm_stamps_read": [_c_void_p, _c_int],
 }
 
 _lib = None

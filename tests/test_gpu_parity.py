@@ -825,6 +825,43 @@ def test_grouped_gemm_headline_problem_set_at_full_depth(ops):
         assert ((c.float() - ref).norm() / ref.norm()).item() <= 1e-2
 
 
+def test_measurement_build_of_the_gemm_kernels_matches_and_stamps_in_order(ops):
+    """The measurement build (time stamps at seven points of every tile) computes what the launched kernels
+    compute, bit for bit, plain and grouped with halves, and every workgroup's stamps are in order."""
+    print("gemm measurement build", flush=True)
+    import ctypes
+    import numpy as np
+    from lego_amd import runtime
+    g = _gen(53)
+    shapes = [(4096, 4096, 128), (4096, 4096, 128), (2048, 4096, 64)]       # 256 + 256 + 128 tiles of 256 x 256: 2.5 rounds
+    A = [(torch.randn(m, k, generator=g) / math.sqrt(k)).half().cuda() for m, n, k in shapes]
+    B = [(torch.randn(k, n, generator=g) / math.sqrt(k)).half().cuda() for m, n, k in shapes]
+    want = _grouped_call("lego_hip_grouped_gemm_f16", A, B)
+    got = _grouped_call("lego_hip_grouped_gemm_f16_stamps", A, B)
+    for c, w in zip(got, want):
+        assert torch.equal(c, w)
+    plan = (ctypes.c_int * 3)()
+    sz = (ctypes.c_int * 9)(*[v for s in shapes for v in s])
+    runtime.call("lego_hip_grouped_gemm_f16_plan", sz, 3, plan)
+    assert plan[0] == 256
+    wgs = plan[1] + plan[2]
+    rows = np.zeros(8 * wgs, dtype=np.uint64)
+    runtime.call("lego_hip_gemm_stamps_read", rows.ctypes.data_as(ctypes.c_void_p), wgs)
+    st = rows.reshape(wgs, 8)[:, :7].astype(np.int64)
+    assert (st[:, 0] > 0).all() and (np.diff(st, axis=1) >= 0).all()
+    a, b = A[0][:1024], B[0][:, :768].contiguous()
+    c0 = torch.empty(1024, 768, dtype=torch.half, device="cuda")
+    c3 = torch.empty_like(c0)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for variant, c in ((0, c0), (3, c3)):
+        runtime.call("lego_hip_gemm_f16_variant", ctypes.c_void_p(a.data_ptr()), ctypes.c_void_p(b.data_ptr()),
+                     ctypes.c_void_p(c.data_ptr()), 1024, 768, 128, variant, stream)
+    torch.cuda.synchronize()
+    assert torch.equal(c0, c3)
+    with pytest.raises(runtime.LegoHipError):
+        runtime.call("lego_hip_gemm_stamps_read", rows.ctypes.data_as(ctypes.c_void_p), 8193)
+
+
 @pytest.mark.parametrize("split", [0, 1, 7, 24, -1])
 def test_grouped_gemm_split_tail_on_ragged_shapes(ops, split):
     """The launch with its last `split` tiles as two halves each, forced through the tuning entry
