@@ -32,6 +32,15 @@ OBJ_DIR = LIB_DIR / "obj"
 # tile's neighbours on all four sides then run on the same XCD at about the same time (measured in one process
 # against column order with non-temporal loads: fp16 9999 x 10001 3.52 -> 4.10 TB/s, 16386 x 8191 2.95 -> 3.92,
 # 10000^2 3.78 -> 4.28; fp32 9999 x 10001 3.79 -> 4.48, 8200 x 8192 3.94 -> 4.89; fp16 10000 x 10240 4.72 -> 4.51).
+# Their macro tiles are 128 bytes of a source row by 512 bytes of a destination row (fp16 256 x 64, fp32 128 x 32): a read
+# segment is one line when it is not cut, a write segment four (five lines touched for four written when it is cut, where
+# the 256-byte segments of the square tiles built before touched three for two).  Against those square tiles, TB/s with
+# rotating results, fp16 any shape 9999 x 10001 4.09 -> 4.23, 8191 x 16386 4.32 -> 4.80, 12345 x 6789 4.14 -> 4.30, 24600 x 24576
+# 4.78 -> 4.95, 16386 x 8191 3.91 -> 3.89; whole vectors 8200 x 8192 4.16 -> 4.47, 10000^2 4.27 -> 4.38, 24600 x 24576 4.86 -> 5.02,
+# 8192 x 8200 4.5 -> 4.44; fp32 any shape 9999 x 10001 4.48 -> 4.60, 16386 x 8191 4.66 -> 4.86, 4099 x 4101 4.18 -> 4.47; whole
+# vectors 10000^2 4.80 -> 5.04, 10000 x 10240 4.91 -> 5.21, 6152^2 4.32 -> 4.65, 8200 x 8192 4.90 -> 4.76, and 24600 x 24576 4.81 ->
+# 4.39, which is why the fp32 tiling with edge tests stops at 384 Mi elements.  Taller or wider tiles lose (fp16 512 x 64:
+# 3.75 at 9999 x 10001; 256 x 128 4.01; 128 x 256 3.68).
 # What remains is the count of 128-byte lines an access touches: the same kernel on fp16 10048^2 (rows of whole lines)
 # moves 5.3 TB/s, on 10016^2 (whole 64-byte halves) 4.5, on 10000^2 3.8 (a 256-byte row segment touches three lines).
 # fp32 4096^2 (2048 workgroups of 32 KiB, five resident per CU: 1.6 rounds) against tilings whose workgroups make whole
@@ -42,17 +51,21 @@ TRANSPOSE = {
             dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("window", 32, 8), max_bytes=1536 << 20),
             dict(dtype="f32", tile=(32, 32), group=(1, 8), order="diag", min_elements=2 << 20),   # smaller: 64x64 tiles
             dict(dtype="f32", tile=(32, 32), group=(2, 2), order="diag"),
+            dict(dtype="f32", tile=(32, 32), group=(4, 1), order=("strip", 8), edge=True, xcd=True, max_elements=384 << 20),
             dict(dtype="f32", tile=(32, 32), group=(2, 4), order=("strip", 8), edge=True, xcd=True),
-            dict(dtype="f32", tile=(32, 32), group=(4, 2), order=("strip", 8), edge=True, ragged=True, xcd=True),
-            dict(dtype="f32", tile=(32, 32), group=(2, 2), order="col", edge=True, ragged=True, xcd=True)],
+            dict(dtype="f32", tile=(32, 32), group=(4, 1), order=("strip", 8), edge=True, ragged=True, xcd=True, min_elements=3 << 20),
+            dict(dtype="f32", tile=(32, 32), group=(2, 2), order="col", edge=True, ragged=True, xcd=True),
+            dict(dtype="f32", tile=(32, 32), group=(4, 2), order=("strip", 8), edge=True, ragged=True, xcd=True, tuning_only=True)],
     "f16": [dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 128, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 64, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order=("window", 32, 8)),
             dict(dtype="f16", tile=(64, 64), group=(1, 4), order="diag", min_elements=2 << 20),   # smaller: 64x64 tiles
             dict(dtype="f16", tile=(64, 64), group=(1, 1), order="diag"),
-            dict(dtype="f16", tile=(64, 64), group=(2, 2), order=("strip", 8), edge=True, xcd=True),
-            dict(dtype="f16", tile=(64, 64), group=(2, 2), order=("strip", 8), edge=True, ragged=True, xcd=True),
-            dict(dtype="f16", tile=(64, 64), group=(1, 1), order="col", edge=True, ragged=True, xcd=True)],
+            dict(dtype="f16", tile=(64, 64), group=(4, 1), order=("strip", 8), edge=True, xcd=True),
+            dict(dtype="f16", tile=(64, 64), group=(4, 1), order=("strip", 8), edge=True, ragged=True, xcd=True, min_elements=40 << 20),
+            dict(dtype="f16", tile=(64, 64), group=(1, 1), order="col", edge=True, ragged=True, xcd=True),
+            dict(dtype="f16", tile=(64, 64), group=(2, 2), order=("strip", 8), edge=True, xcd=True, tuning_only=True),
+            dict(dtype="f16", tile=(64, 64), group=(2, 2), order=("strip", 8), edge=True, ragged=True, xcd=True, tuning_only=True)],
 }
 # (element type, vectorised, waves per row): 16-byte accesses need N % (16/size) == 0; the
 # element-per-access kernels ("s") take any N
@@ -97,6 +110,7 @@ def collect():
             max_bytes = cfg.pop("max_bytes", None)   # only for matrices that fit the last-level cache
             tuning_only = cfg.pop("tuning_only", False)      # built for comparison, never picked
             min_elements = cfg.pop("min_elements", None)
+            max_elements = cfg.pop("max_elements", None)
             unit, meta = transpose.emit(**cfg)
             meta["max_bytes"] = max_bytes
             meta["tuning_only"] = tuning_only
@@ -108,14 +122,16 @@ def collect():
                 # smaller matrices have too few of these macro tiles: the 64x64 ones of the any-shape kernels are ahead up
                 # to about 32 Mi elements (fp16 2056^2 3.2 against 2.3 TB/s, 4104^2 4.2 / 3.8; 6152^2 3.7 / 4.0)
                 meta["min_elements"] = 32 << 20
+            meta["max_elements"] = max_elements
             meta["any_element"] = bool(cfg.get("ragged"))
             if cfg.get("ragged"):     # any shape with at least one whole vector per row of both matrices
                 meta["row_multiple"] = meta["col_multiple"] = 1
                 meta["min_side"] = vec
-                # 64x64 tiles up to 64 Mi elements (fp16 4099 x 4101: 3.9 against 3.1 TB/s with 128x128 tiles, 6001 x 6003 3.5
-                # against 3.3), the larger tile above (9999 x 10001: 3.5 against 3.4); matrices of under 16 Ki elements
-                # go one element per access
-                meta["min_elements"] = (64 << 20) if meta["SR"] * meta["SC"] > 64 * 64 else (16 << 10)
+                # 64x64 tiles for the smaller matrices, which have too few of the larger macro tiles: fp16 up to 40 Mi
+                # elements (64x64 / 256x64, TB/s: 4099 x 4101 3.69 / 3.45, 6001 x 6003 3.94 / 3.81, 7001 x 7003 3.94 / 4.02),
+                # fp32 up to 3 Mi (64x64 / 128x32: 1449 x 1451 2.49 / 2.40, 2049 x 2051 3.29 / 3.41, 4099 x 4101 4.15 / 4.47);
+                # matrices of under 16 Ki elements go one element per access
+                meta["min_elements"] = (min_elements or (64 << 20)) if (meta["SR"], meta["SC"]) != (64, 64) else (16 << 10)
             unit.filename = meta["kernel"].replace("lego_", "", 1) + ".hip"
             units.append(unit)
             tmeta.setdefault(dtype, []).append(meta)
@@ -182,6 +198,8 @@ def collect():
                 fits += f" && rows >= {m['min_side']} && cols >= {m['min_side']}"
             if m.get("min_elements"):
                 fits += f" && 1ull * rows * cols >= {m['min_elements']}ull"
+            if m.get("max_elements"):
+                fits += f" && 1ull * rows * cols <= {m['max_elements']}ull"
             h.append(f"  if (rows % {m['row_multiple']} == 0 && cols % {m['col_multiple']} == 0{fits}) "
                      f"return {m['kernel']}_launch(in, out, rows, cols, stream);")
         h += [f"  return lego_transpose_any_launch(in, out, rows, cols, {4 if dtype == 'f32' else 2}, stream);", "}",
@@ -189,7 +207,7 @@ def collect():
               f"inline hipError_t lego_transpose_{dtype}_dispatch_any_base(const void* in, void* out, int rows, int cols, "
               "hipStream_t stream) {"]
         for m in metas:
-            if m["any_element"]:
+            if m["any_element"] and not m["tuning_only"]:
                 h.append(f"  if (rows >= {m['min_side']} && cols >= {m['min_side']} && 1ull * rows * cols >= {m['min_elements']}ull) "
                          f"return {m['kernel']}_launch(in, out, rows, cols, stream);")
         h += [f"  return lego_transpose_any_launch(in, out, rows, cols, {4 if dtype == 'f32' else 2}, stream);", "}",
