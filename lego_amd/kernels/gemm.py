@@ -453,6 +453,8 @@ def _tile_params(bm, bn, bk, waves, max_group_m, trans_a, trans_b, with_grouped,
         banner=BANNER, elt=elt, out_elt=out_elt, ESIZE=esize, EPC=EPC, MFMA_K=mfma_k, NPH=NPH,
         FMT={"e4m3": 0, "e5m2": 1}.get(dtype, 0), dt=dtype, mfma_dt={"bf16h": "bf16"}.get(dtype, dtype), BM=bm, BN=bn, BK=bk, THREADS=THREADS, WAVES_M=WAVES_M, WAVES_N=WAVES_N,
         WM=WM, WN=WN, TM=TM, TN=TN, A_ITERS=A_ITERS, B_ITERS=B_ITERS, DMA_LAST=DMA_LAST,
+        # s_waitcnt immediate: vmcnt in bits 3:0 and 15:14, expcnt and lgkmcnt left at their maxima
+        WAIT_DMA_LAST="0x%04X" % (0x0F70 | (DMA_LAST % 16) | ((DMA_LAST // 16) << 14)),
         load_slots=load_slots, dma_last=dma_last, dma_first=dma_first, dma_none=none, XCDS=XCDS, MAX_GROUPS=MAX_GROUPS,
         last_slots=last_slots, last_tail=last_tail, RING=LAST_KTILE_RING,
         pid_layout="OrderBy(Col(max(npm//GM,1),1), Col(min(npm,GM),npn)).TileBy([npm,npn]).inv(pid)",
