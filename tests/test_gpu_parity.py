@@ -262,10 +262,12 @@ def test_layernorm_ragged_and_fp32(ops, dtype, M, N):
         assert torch.allclose(rstd.cpu(), want_rstd, atol=1e-4, rtol=1e-3)
 
 
-@pytest.mark.parametrize("M,N", [(24600, 8191), (201500, 1001)])
+@pytest.mark.parametrize("M,N", [(24600, 8191), (201500, 1001), (16386, 8191), (65541, 781), (33000, 6152)])
 def test_rows_of_any_length_in_several_launches(ops, M, N):
-    """Tall matrices of rows of any length: the walking kernels run in launches of at most 16 rows per team, one
-    after the other.  At this size:
+    """Tall matrices of rows of any length: the walking kernels run in launches of about 16 rows per team (64 for rows
+    of whole vectors), one after the other, equal in length, and a remainder of under a quarter of a launch is folded
+    into the launches before it (16386 x 8191: launches of 8704 and 7682 rows; 65541 x 781: one launch of 17 steps;
+    33000 x 6152, rows of whole vectors: one launch of 65 steps).  At this size:
     row sums of the softmax, the statistics against torch on the GPU, and the first and last rows (the ends of
     the first and of the last launch) against the oracle."""
     print(f"rows of any length, large result {M}x{N}", flush=True)
@@ -280,7 +282,7 @@ def test_rows_of_any_length_in_several_launches(ops, M, N):
     assert (mean - xf.mean(-1)).abs().max().item() <= 1e-4
     assert ((rstd - torch.rsqrt(xf.var(-1, unbiased=False) + 1e-5)).abs() <= 1e-3 * rstd.abs()).all()
     del xf
-    for rows in (slice(0, 48), slice(M // 2 - 24, M // 2 + 24), slice(M - 48, M)):
+    for rows in (slice(0, 48), slice(M // 2 - 24, M // 2 + 24), slice(M - 48, M), slice(8704 - 24, 8704 + 24)):
         x = xd[rows].cpu()
         assert (sm[rows].cpu().float() - ok.softmax(x).float()).abs().max().item() <= TOL
         _assert_layernorm_forward(y[rows], x, w, b)
