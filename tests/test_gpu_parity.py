@@ -1258,3 +1258,14 @@ def test_gemm_leaky_relu_epilogue(ops):
     assert _rel_err(got, want) <= 1e-2
     assert (got.float() - want.float()).abs().max().item() <= 1e-2
     assert (got < 0).any() and (got > 0).any()
+
+
+def test_tuner_compares_the_alternatives(ops, capsys):
+    """`python -m lego_amd.tune`: every alternative behind a dispatch threshold through its tuning entry point."""
+    print("tuner", flush=True)
+    from lego_amd import tune
+    assert tune.main(["transpose", "--dtype", "f32", "--shapes", "1000x1004"]) == 0
+    assert tune.main(["rows", "--shapes", "512x1024"]) == 0
+    assert tune.main(["gemm", "--shapes", "512x512x256"]) == 0
+    out = capsys.readouterr().out
+    assert "dispatch:" in out and "ragged" in out and "4 waves:" in out and "16x16x32, 4 waves:" in out
