@@ -487,10 +487,20 @@ def main():
             ref8 = a8[:256].float() @ b8.float()
             rel8 = ((c8[:256].float() - ref8).norm() / ref8.norm()).item()
             ms8 = timed(g8f, steps=max(5, K // 5), warmup=max(2, W // 5))
+            # the same instruction with nothing around it, on operands of the same distribution
+            ops8 = a8.view(-1)[:probe_wgs * 65536]
+            ms_probe8 = timed(lambda: runtime.call("lego_hip_mfma_probe", p(ops8), p(probe_sink), 5, probe_iters // 2, probe_wgs, stream),
+                              steps=max(5, K // 5), warmup=max(2, W // 5))
+            ceiling8 = probe_wgs * (probe_iters // 2) * 8388608.0 / ms_probe8 / 1e9
+            kernels["mfma_ceiling_fp8_e5m2"] = dict(
+                ms=ms_probe8, tflops=ceiling8, frac_mfma=ceiling8 / MFMA_FP8_PEAK_TFLOPS,
+                note="v_mfma_f32_32x32x64_f8f6f4 only, operands randn cast to e5m2 held in registers, 256 workgroups of "
+                     "four waves: what the part sustains with the pipe full")
             kernels["next_gemm_fp8_e5m2_8192"] = dict(ms=ms8, tflops=fl4 / ms8 / 1e9,
                                                       frac_mfma=fl4 / ms8 / 1e9 / MFMA_FP8_PEAK_TFLOPS,
+                                                      achievable_tflops=ceiling8, frac_of_achievable=fl4 / ms8 / 1e9 / ceiling8,
                                                       rel_err_vs_fp32=rel8, note="peak = 5.0 PFLOP/s dense fp8")
-            del a8, b8, c8, ref8
+            del a8, b8, c8, ref8, ops8
             # shapes off the tile grid: ragged in M and N (lane masks in scalar registers instead of edge tests), and
             # a skinny product split along K with a workspace (bound by reading B once: GB/s of operand bytes)
             mr = nr = 8184

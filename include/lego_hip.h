@@ -295,6 +295,8 @@ int lego_hip_hbm_probe(const void* in, void* out, unsigned long long bytes, int 
  *   shape 2: v_mfma_f32_32x32x16_bf16 (the same bits read as bfloat16; flop as shape 0)
  *   shape 3 / 4: the instructions of shapes 1 / 0 with two waves per SIMD (workgroups of eight waves with 128
  *   accumulator registers each, a 128 x 64 block per wave: 4194304 / 2097152 flop per round and workgroup).
+ *   shape 5 / 6: v_mfma_f32_32x32x64_f8f6f4 with the operands' bytes read as OCP e5m2 / e4m3 (16 per round and
+ *   wave over 4 x 4 blocks: 8388608 flop per round and workgroup; the same workgroups * 64 KiB of operands).
  * sink: workgroups * 512 floats (a sum per lane, so that the work is not optimised away).  bench.py runs it with
  * operands of the GEMM benchmark's distribution and reports the rate as what the socket's power limit leaves to
  * an fp16 GEMM whose data movement costs nothing. */

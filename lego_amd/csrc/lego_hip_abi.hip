@@ -196,6 +196,39 @@ __global__ void __launch_bounds__(256) lego_mfma_probe_kernel(const probe_half8*
   sink[static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x] = total;
 }
 
+// 8-bit operands: v_mfma_f32_32x32x64_f8f6f4 on 4 x 4 blocks, the operands' bits read as OCP e5m2 (shape 5) or e4m3 (6)
+typedef int probe_int8 __attribute__((ext_vector_type(8)));
+template <int FORMAT>     // 0: e4m3  1: e5m2 (the instruction's format codes)
+__global__ void __launch_bounds__(256) lego_mfma_probe_8bit_kernel(const probe_int8* __restrict__ operands, float* __restrict__ sink, unsigned iters)
+{
+  const probe_int8* mine = operands + (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 8;
+  probe_int8 fa[4], fb[4];
+#pragma unroll
+  for (int f = 0; f < 4; ++f) { fa[f] = mine[f]; fb[f] = mine[4 + f]; }
+  probe_float16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  for (unsigned it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[j], fa[i], acc[i][j], FORMAT, FORMAT, 0, 0, 0, 0);
+  }
+  float total = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) total += acc[i][j][r];
+  sink[static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x] = total;
+}
+
 typedef unsigned u32x4w __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4w_any __attribute__((ext_vector_type(4), aligned(2)));     // the same 16 bytes at any 2-byte element
 
@@ -1109,11 +1142,13 @@ int lego_hip_hbm_probe(const void* in, void* out, unsigned long long bytes, int 
 
 int lego_hip_mfma_probe(const void* operands, float* sink, int shape, int iters, int workgroups, void* stream)
 {
-  if (!usable(operands) || !usable(sink) || shape < 0 || shape > 4 || iters <= 0 || workgroups <= 0) return kInvalid;
+  if (!usable(operands) || !usable(sink) || shape < 0 || shape > 6 || iters <= 0 || workgroups <= 0) return kInvalid;
   const dim3 grid(static_cast<unsigned>(workgroups)), block(256);
   const probe_half8* src = static_cast<const probe_half8*>(operands);
   hipStream_t s = as_stream(stream);
-  if (shape == 3) hipLaunchKernelGGL(lego_mfma_probe2_kernel<3>, grid, dim3(512), 0, s, src, sink, static_cast<unsigned>(iters));
+  if (shape == 5) hipLaunchKernelGGL(lego_mfma_probe_8bit_kernel<1>, grid, block, 0, s, static_cast<const probe_int8*>(operands), sink, static_cast<unsigned>(iters));
+  else if (shape == 6) hipLaunchKernelGGL(lego_mfma_probe_8bit_kernel<0>, grid, block, 0, s, static_cast<const probe_int8*>(operands), sink, static_cast<unsigned>(iters));
+  else if (shape == 3) hipLaunchKernelGGL(lego_mfma_probe2_kernel<3>, grid, dim3(512), 0, s, src, sink, static_cast<unsigned>(iters));
   else if (shape == 4) hipLaunchKernelGGL(lego_mfma_probe2_kernel<4>, grid, dim3(512), 0, s, src, sink, static_cast<unsigned>(iters));
   else if (shape == 0) hipLaunchKernelGGL(lego_mfma_probe_kernel<0>, grid, block, 0, s, src, sink, static_cast<unsigned>(iters));
   else if (shape == 1) hipLaunchKernelGGL(lego_mfma_probe_kernel<1>, grid, block, 0, s, src, sink, static_cast<unsigned>(iters));
