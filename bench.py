@@ -44,7 +44,7 @@ def headline_traffic_bytes():
     try:
         with open(TRAFFIC_PROFILE) as fh:
             for line in fh:
-                if line.startswith(HEADLINE_KERNEL + " "):
+                if line.startswith((HEADLINE_KERNEL + " ", HEADLINE_KERNEL + "<")):
                     numbers = [int(tok) for tok in line.split(")", 1)[1].split() if tok.isdigit()]
                     return numbers[2]          # fetch KiB, write KiB, scaled bytes, algorithmic
     except (OSError, IndexError, ValueError):

@@ -24,6 +24,7 @@ from ..lego import BitXor, Col, GenP, OrderBy, Row  # noqa: F401
 from .common import BANNER, Emitted, code, idx, size, template, tidy
 
 THREADS = 256
+FEW_RESIDENT_FROM = 4096     # macro tiles of a launch from which three resident workgroups per CU are ahead of four or five
 
 
 def lane_block(esize):
@@ -222,6 +223,8 @@ def emit(dtype="f32", tile=(32, 32), group=(2, 2), order="row", suffix="", edge=
         dst_off0=code(in_tile(dst, rv * rows_per_read, k * cols_per_word, rng2)),
         dst_off1=code(in_tile(dst, rv * rows_per_read, k * cols_per_word + 1, rng2)) if esize == 2 else "",
         xcd=xcd,
+        # whole-tile kernels: from FEW_FROM macro tiles on, an LDS footprint that leaves three workgroups on a CU
+        FEW_FROM=FEW_RESIDENT_FROM, FEW_LDS_BYTES=163840 // 3 // 1024 * 1024,
         grid=(f"(static_cast<unsigned>((rows + {SR - 1}) / {SR}) * static_cast<unsigned>((cols + {SC - 1}) / {SC}) + 7) / 8 * 8" if edge and xcd else
               f"static_cast<unsigned>((rows + {SR - 1}) / {SR}) * static_cast<unsigned>((cols + {SC - 1}) / {SC})" if edge
               else f"static_cast<unsigned>(rows / {SR}) * static_cast<unsigned>(cols / {SC})"),
