@@ -38,7 +38,7 @@ def test_benchmark_reads_the_committed_traffic_summary():
     import bench
     got = bench.headline_traffic_bytes()
     text = open(bench.TRAFFIC_PROFILE).read()
-    row = next(line for line in text.splitlines() if line.startswith(bench.HEADLINE_KERNEL + " "))
+    row = next(line for line in text.splitlines() if line.startswith((bench.HEADLINE_KERNEL + " ", bench.HEADLINE_KERNEL + "<")))
     fetch_kib, write_kib, scaled, algorithmic = [int(t) for t in row.split(")", 1)[1].split()[:4]]
     assert got == scaled
     # the scaled figure is what the counters say, each scaled by what the same counter reads for the plain
