@@ -77,12 +77,16 @@ ROWWISE = [("f16", True, 1), ("f16", True, 2), ("f16", True, 4), ("f16", True, 8
 # (element type, lanes per row): teams of a part of a wave for rows of at most that many 16-byte vectors
 ROWWISE_SHORT = [(d, lanes, vec) for d in ("f16", "bf16", "f32") for lanes in (16, 32) for vec in (True, False)]
 # LayerNorm launches of many rows: this many workgroups that stage gamma and beta in LDS and walk the rows
-ROWWISE_STREAM_WGS = {("f16", True, 8): 512, ("bf16", True, 8): 512, ("f32", True, 8): 512, ("f16", True, 16): 256, ("bf16", True, 16): 256,
+ROWWISE_STREAM_WGS = {("f16", True, 4): 1024, ("bf16", True, 4): 1024, ("f16", True, 8): 512, ("bf16", True, 8): 512, ("f32", True, 8): 512, ("f16", True, 16): 256, ("bf16", True, 16): 256,
                       # rows of any length: a team's rows must start alike, so the count times the teams per workgroup is a multiple of 8
                       ("f16", False, 1): 1024, ("f16", False, 4): 1024, ("f16", False, 16): 256,
                       ("f16", False, 8): 512, ("bf16", False, 8): 512, ("f32", False, 8): 512,
                       ("bf16", False, 1): 1024, ("bf16", False, 4): 1024, ("bf16", False, 16): 256,
                       ("f32", False, 1): 1024, ("f32", False, 4): 1024, ("f32", False, 16): 256}
+# ... of teams of four waves only with four vectors per lane (16-bit rows of 4097-8192 elements); measured with and without
+# the walking launch, fp16 TB/s: 8192 x 5120 5.22 / 5.47, 8192 x 6144 5.48 / 5.57, 2048 x 8192 5.01 / 5.39, but
+# 8192 x 3072 5.13 / 4.96, 16384 x 4096 5.89 / 5.81, 65536 x 2560 6.07 / 5.47
+ROWWISE_STREAM_MIN_VECTORS = {("f16", True, 4): 4, ("bf16", True, 4): 4}
 ROWWISE_DEFAULT_WAVES = 4
 ROWWISE_WIDE_TEAM_ABOVE_N, ROWWISE_WIDE_TEAM_FROM_M = 6144, 4096
 ROWWISE_MAX_N = rowwise.MAX_N
@@ -136,7 +140,8 @@ def collect():
             units.append(unit)
             tmeta.setdefault(dtype, []).append(meta)
     units.append(transpose.emit_any())
-    units += [rowwise.emit(w, dtype, vec, stream_wgs=ROWWISE_STREAM_WGS.get((dtype, vec, w), 0)) for dtype, vec, w in ROWWISE]
+    units += [rowwise.emit(w, dtype, vec, stream_wgs=ROWWISE_STREAM_WGS.get((dtype, vec, w), 0),
+                           stream_min_vectors=ROWWISE_STREAM_MIN_VECTORS.get((dtype, vec, w), 1)) for dtype, vec, w in ROWWISE]
     units += [rowwise.emit(1, dtype, vec, team_lanes=lanes) for dtype, lanes, vec in ROWWISE_SHORT]
     units.append(rowwise.emit_long())
     for dtype in GEMM_DTYPES:

@@ -27,13 +27,16 @@ LONG_ROW_WAVES = 16
 VPTS = (1, 2, 4, 8, 16, 32, 64)
 
 
-def emit(waves_per_row=1, dtype="f16", vectorised=True, seq_max_wpr=4, prefetch_max_wpr=4, stream_wgs=0, team_lanes=None):
+def emit(waves_per_row=1, dtype="f16", vectorised=True, seq_max_wpr=4, prefetch_max_wpr=4, stream_wgs=0, team_lanes=None,
+         stream_min_vectors=1):
     """One translation unit: every register footprint ``V`` of one (waves per row, element type,
     access width) combination.  ``vectorised=False`` emits the kernels that take rows of any length
     and alignment (the reference's own softmax test is 1823 x 781): the elements before a row's
     first 16-byte boundary and after its last whole vector go one per lane, the rest as vectors.
     ``team_lanes`` (16 or 32) makes teams of a part of a wave for rows of at most ``team_lanes`` vectors:
-    a row of 128 halves in a wave of its own would leave 48 of 64 lanes without a vector."""
+    a row of 128 halves in a wave of its own would leave 48 of 64 lanes without a vector.
+    ``stream_wgs`` workgroups walk the rows of a LayerNorm launch of many rows (0: no such launch), for the
+    register footprints of at least ``stream_min_vectors`` vectors per lane."""
     WPR = waves_per_row
     elt, esize = ELEMENTS[dtype]
     EPV = 16 // esize
@@ -76,7 +79,7 @@ def emit(waves_per_row=1, dtype="f16", vectorised=True, seq_max_wpr=4, prefetch_
         VPTS=[1] if team_lanes else [vp for vp in VPTS if vp * EPV <= 128 and lo < vp * TEAM * EPV <= hi],
         dtype=dtype, elt=elt, EPV=EPV, ESIZE=esize, RAGGED=not vectorised, tag=tag,
         SEQ_MAX_WPR=seq_max_wpr, PREFETCH_MAX_WPR=prefetch_max_wpr,
-        STREAM=stream_wgs > 0 and (RPW == 1 or not vectorised), STREAM_WGS=stream_wgs,
+        STREAM=stream_wgs > 0 and (RPW == 1 or not vectorised), STREAM_WGS=stream_wgs, STREAM_MIN_V=stream_min_vectors,
         WALK_STEPS=64 if vectorised else 16,     # rows per team and launch of the walking kernels
         stream_team_layout=f"OrderBy(Row(STEPS, G, {RPW})).TileBy([STEPS], [G], [{RPW}])[step, wg, team]",
         stream_team_row=code(stream_team_row), stream_team0_row=code(stream_team0_row),
