@@ -317,7 +317,9 @@ def test_layernorm_fp32_long_rows_through_the_c_abi(ops, N):
 # 600 and 515 rows of more than 16384 elements: the same walk with sixteen waves, one row across 1024 lanes
 @pytest.mark.parametrize("M,N", [(7, 8), (33, 520), (64, 1024), (129, 4096), (1151, 8192), (3, 16384), (4100, 8200),
                                  (1030, 16384), (600, 32768), (515, 20488), (511, 32768),
-                                 (2500, 3080)])     # one round of workgroups: the default takes teams of two waves
+                                 (2500, 3080),      # one round of workgroups: the default takes teams of two waves
+                                 # teams of four waves with four vectors per lane walk rows as well (from 2048 rows on)
+                                 (2050, 5128), (2049, 8192)])
 def test_layernorm_matches_oracle(ops, M, N, wpr):
     print(f"layernorm {M}x{N} wpr={wpr}", flush=True)
     if wpr is not None and N > min(8192 * wpr, 16384):
