@@ -89,6 +89,7 @@ ROWWISE_STREAM_WGS = {("f16", True, 4): 1024, ("bf16", True, 4): 1024, ("f16", T
 ROWWISE_STREAM_MIN_VECTORS = {("f16", True, 4): 4, ("bf16", True, 4): 4}
 ROWWISE_DEFAULT_WAVES = 4
 ROWWISE_WIDE_TEAM_ABOVE_N, ROWWISE_WIDE_TEAM_FROM_M = 6144, 4096
+ROWWISE_TWO_WAVES_ABOVE_N, ROWWISE_TWO_WAVES_FROM_M = 1536, 16384
 ROWWISE_MAX_N = rowwise.MAX_N
 GEMM = dict(bm=256, bn=256, bk=64, waves=(2, 2), max_group_m=8)
 GEMM_SMALL_TILE = 128
@@ -247,9 +248,11 @@ def collect():
           "// rows of tall matrices, where they measure 3-5 % above four waves; fewer rows leave too few workgroups",
           "// ... and two waves (two rows per workgroup) for 2049-4096 rows of 2049-4096 elements: one round of workgroups on",
           "// the 256 CUs instead of two (4096 x 4096: softmax 4.9 -> 5.4 TB/s, LayerNorm 4.4 -> 5.0; no gain from 8192 rows on)",
+          "// ... and for rows of 1537-2048 elements, which one wave holds as four vectors per lane, of matrices of 16384 rows",
+          "// and more (2-5 % above one wave there, 1-11 % below it at 8192 rows)",
           f"inline int lego_rowwise_f16_wpr(int m, int n) {{ return n > {ROWWISE_WIDE_TEAM_ABOVE_N} && n <= "
           f"{rowwise.MAX_N_SMALL_TEAMS} && m >= {ROWWISE_WIDE_TEAM_FROM_M} ? 8 : n > 2048 && n <= 4096 && m > 2048 && m <= 4096 ? 2 "
-          ": lego_rowwise_default_wpr(n); }", ""]
+          f": n > {ROWWISE_TWO_WAVES_ABOVE_N} && n <= 2048 && m >= {ROWWISE_TWO_WAVES_FROM_M} ? 2 : lego_rowwise_default_wpr(n); }}", ""]
     h += ["unsigned lego_layernorm_bwd_groups(int M, int N);", "unsigned lego_layernorm_bwd_f32_groups(int M, int N);",
           "unsigned lego_layernorm_bwd_bf16_groups(int M, int N);",
           "hipError_t lego_layernorm_bwd_f32_launch(const void*, const void*, const void*, const float*, const float*, "

@@ -171,7 +171,8 @@ def _assert_layernorm_forward(y, x, w, b, eps=1e-5):
 @pytest.mark.parametrize("wpr", [None, 1, 2, 4, 8])
 @pytest.mark.parametrize("M,N", [(7, 8), (33, 520), (64, 1024), (5, 2048), (129, 4096), (16, 8192), (3, 16384),
                                  (4100, 8200),      # tall and long: the default takes teams of eight waves
-                                 (2500, 3080)])     # one round of workgroups: the default takes teams of two
+                                 (2500, 3080),      # one round of workgroups: the default takes teams of two
+                                 (16390, 1600)])    # very tall, four vectors per lane of one wave: teams of two as well
 def test_softmax_matches_oracle(ops, M, N, wpr):
     print(f"softmax {M}x{N} wpr={wpr}", flush=True)
     if wpr is not None and N > min(8192 * wpr, 16384):
@@ -319,7 +320,8 @@ def test_layernorm_fp32_long_rows_through_the_c_abi(ops, N):
                                  (1030, 16384), (600, 32768), (515, 20488), (511, 32768),
                                  (2500, 3080),      # one round of workgroups: the default takes teams of two waves
                                  # teams of four waves with four vectors per lane walk rows as well (from 2048 rows on)
-                                 (2050, 5128), (2049, 8192)])
+                                 (2050, 5128), (2049, 8192),
+                                 (16390, 1600)])    # very tall, four vectors per lane of one wave: the default takes two waves
 def test_layernorm_matches_oracle(ops, M, N, wpr):
     print(f"layernorm {M}x{N} wpr={wpr}", flush=True)
     if wpr is not None and N > min(8192 * wpr, 16384):
