@@ -599,20 +599,38 @@ typedef hipError_t (*gemm_launcher)(const void*, const void*, void*, int, int, i
 struct GemmKernels {
   gemm_launcher big[4];     // 256 x 256 tiles, one workgroup per CU; index 2*trans_a + trans_b
   gemm_launcher small[4];   // 128 x 128 tiles, two workgroups per CU (null: not built for this type)
+  gemm_launcher sparse[4];  // 256 x 256 tiles on 32x32x16 MFMAs, for launches that leave many CUs idle (null: not built)
 };
 // Fewer 256 x 256 tiles than this and the 128 x 128 kernel, with four times as many workgroups,
 // keeps more of the 256 CUs busy than its higher LDS traffic per flop costs.
 constexpr long kSmallTileBelow = 129;
-// The same for larger products whose 256 x 256 tiles leave the last round of workgroups mostly empty: the share of
-// workgroup slots that do work, over whole rounds of 256 (512 for the small tile, which runs at about 0.8 of the
-// large tile's rate), decides.  4608^3, 324 tiles in two rounds: 0.98 -> 1.02 PFLOP/s; 5120^3 and 6144^3 stay.
+// One round of 256 x 256 tiles that leaves this many CUs or more without a tile runs faster on the 32x32x16 MFMA: away
+// from the socket's power limit its fewer LDS reads per flop count for more than the 16x16x32's lower energy per flop
+// (fp16, 144 tiles: 0.95 -> 1.02 PFLOP/s at 2304 x 4096 x 4096, 0.75 -> 0.85 at 3072 x 3072 x 1024; 160 tiles 1.05 -> 1.08;
+// 176 tiles 1.08 -> 1.09; 192 tiles 1.16 -> 1.14).
+constexpr long kSparseRoundBelow = 176;
+// Time of a last round in which only `share` of the workgroup slots hold a tile, in units of a full round.  A few busy
+// CUs run at the clock that the socket's power limit denies the full chip, so the round is shorter than a full one
+// even though each of its tiles takes a CU to itself.
+inline double partial_round(double share, double least, double knee)
+{
+  if (share <= 0.0) return 0.0;
+  return share <= knee ? least : least + (share - knee) * (1.0 - least) / (1.0 - knee);
+}
+// Larger products whose 256 x 256 tiles leave the last round of workgroups mostly empty take the small tile when the
+// estimate of its time is the lower one: whole rounds of 256 big or 512 small tiles (the small tile runs at about 0.8
+// of the large tile's rate, so a round of it costs 0.625 of a big one) plus the partial last round.  Measured on fp16
+// products 4096 deep, time of a round of big tiles by the share of CUs it keeps busy: 0.06-0.5 -> 0.69-0.71, 0.56 ->
+// 0.76, 0.69 -> 0.82, 0.81 -> 0.88, 0.94 -> 0.97; of small tiles: 0.13 -> 0.51, 0.5 -> 0.58.  4352 x 4096 x 4096 (272
+// tiles): 0.81 big, 0.87 small; 5120 x 4096 (320): 0.95 / 1.00; 4608^3 (324): 0.98 / 1.02; 6144 x 4096 (384, a half
+// round left over): 1.13 / 1.04; 5120^3 and 6144^3 stay with the big tile.
 inline bool small_tiles_fill_better(int M, int N, long tiles)
 {
   if (tiles < kSmallTileBelow) return true;
   const long small = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
-  const double fill_big = static_cast<double>(tiles) / (256 * ((tiles + 255) / 256));
-  const double fill_small = static_cast<double>(small) / (512 * ((small + 511) / 512));
-  return 0.8 * fill_small > fill_big;
+  const double big_time = static_cast<double>(tiles / 256) + partial_round(static_cast<double>(tiles % 256) / 256.0, 0.69, 0.5);
+  const double small_time = 0.625 * (static_cast<double>(small / 512) + partial_round(static_cast<double>(small % 512) / 512.0, 0.5, 0.4));
+  return small_time < big_time;
 }
 
 int gemm_ex(const GemmKernels& k, int element, const void* a, const void* b, void* c, int M, int N, int K,
@@ -637,7 +655,8 @@ int gemm_ex(const GemmKernels& k, int element, const void* a, const void* b, voi
   }
   const long tiles = static_cast<long>((M + LEGO_GEMM_BM - 1) / LEGO_GEMM_BM) * ((N + LEGO_GEMM_BN - 1) / LEGO_GEMM_BN);
   const int layout = (trans_a ? 2 : 0) + (trans_b ? 1 : 0);
-  const gemm_launcher* by_layout = small_tiles_fill_better(M, N, tiles) && k.small[layout] != nullptr ? k.small : k.big;
+  const gemm_launcher* by_layout = small_tiles_fill_better(M, N, tiles) && k.small[layout] != nullptr ? k.small
+                                   : tiles < kSparseRoundBelow && k.sparse[layout] != nullptr ? k.sparse : k.big;
   return ok_or(by_layout[layout](a, b, c, M, N, K, activation, as_stream(stream)));
 }
 
@@ -671,7 +690,11 @@ typedef hipError_t (*splitk_launcher)(const void*, const void*, void*, int, int,
 int lego_hip_gemm_f16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                          int activation, void* stream)
 {
-  static const GemmKernels k = LEGO_GEMM_KERNELS(f16);
+  static const GemmKernels k = [] {
+    GemmKernels t = LEGO_GEMM_KERNELS(f16);
+    t.sparse[0] = lego_gemm_f16_nn_m32_launch;      // built for operands as given only
+    return t;
+  }();
   return gemm_ex(k, 0, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
 }
 

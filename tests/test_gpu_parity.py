@@ -559,6 +559,42 @@ def test_gemm_integer_exact(ops):
     assert torch.equal(got.double(), want)
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (300, 264, 72), (1000, 520, 136), (512, 768, 256)])
+def test_gemm_on_32x32x16_mfmas_is_exact_on_small_integers(ops, M, N, K):
+    """The build of the 256 x 256-tile kernel on the 32x32x16 MFMA (taken by launches that leave many CUs without a
+    tile), through its tuning entry point: whole and ragged tiles, a ragged last k-tile, bit for bit."""
+    print(f"gemm on 32x32x16 MFMAs {M}x{N}x{K}", flush=True)
+    import ctypes
+    from lego_amd import runtime
+    g = _gen(71)
+    a = torch.randint(-2, 3, (M, K), generator=g).half()
+    b = torch.randint(-2, 3, (K, N), generator=g).half()
+    ad, bd = a.cuda(), b.cuda()
+    c = torch.full((M, N), float("nan"), dtype=torch.half, device="cuda")
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    runtime.call("lego_hip_gemm_f16_variant", p(ad), p(bd), p(c), M, N, K, 1, None)
+    torch.cuda.synchronize()
+    assert torch.equal(c.cpu().double(), a.double() @ b.double())
+
+
+@pytest.mark.parametrize("M,N,K", [(2304, 4096, 64), (2300, 4088, 72), (3072, 3072, 128), (2560, 4096, 64),
+                                   # a half round left over: big tiles by the estimate of the launch's time
+                                   (6144, 4096, 64), (4352, 4096, 64)])
+def test_gemm_launches_that_leave_cus_idle(ops, M, N, K):
+    """129 to 175 tiles of 256 x 256 (one round that leaves a third of the CUs idle) take the 32x32x16 build, with
+    and without the fused activation; products of one and a half rounds choose between the tile sizes by estimate.
+    Small integers: bit for bit."""
+    print(f"gemm sparse round {M}x{N}x{K}", flush=True)
+    g = _gen(72)
+    a = torch.randint(-2, 3, (M, K), generator=g).half()
+    b = torch.randint(-2, 3, (K, N), generator=g).half()
+    want = a.float() @ b.float()                       # |sums| <= 4 * 128: exact in fp32 and fp16
+    ad, bd = a.cuda(), b.cuda()
+    assert torch.equal(ops.matmul(ad, bd).cpu().float(), want)
+    act = ops.matmul(ad, bd, activation="leaky_relu").cpu()
+    assert torch.equal(act, torch.where(want >= 0, want, 0.01 * want).half())
+
+
 def test_grouped_gemm_matches_oracle(ops):
     print("grouped gemm", flush=True)
     g = _gen(5)
