@@ -97,6 +97,7 @@ GEMM_WAVES_TWO_PER_SIMD = (2, 4)
 GEMM_SMALL_DTYPES = ("f16", "bf16", "bf16h")     # a 128-byte row of 8-bit elements is too short for their [k][n] rotation
 GEMM_SMALL_NT_ONLY = ("e4m3", "e5m2")             # ... so 8-bit operands get the small tile where both are k-major (A as given, B transposed)
 GEMM_DTYPES = ("f16", "bf16", "bf16h", "e4m3", "e5m2")     # bf16h: bfloat16 operands, fp16 result
+GEMM_SPARSE_ROUND_DTYPES = ("f16", "bf16", "bf16h")   # 16-bit operands: also built on the 32x32x16 MFMA (see collect())
 # The MFMA of the 256 x 256 tiles: v_mfma_f32_16x16x32 for 16-bit operands (the same matrix-core cycles per flop as
 # 32x32x16, but the socket's power limit leaves it a higher clock: a stream of nothing but MFMAs runs 1.95 against
 # 1.68 PFLOP/s, and the GEMM gains 3 to 7 %: 8192^3 1.29 -> 1.36, 4096^3 1.22 -> 1.31, 8192 x 8192 x 1024 1.12 -> 1.17
@@ -165,18 +166,21 @@ def collect():
                     gs, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK[dtype], bm=GEMM_SMALL_TILE, bn=GEMM_SMALL_TILE),
                                       trans_a=ta, trans_b=tb, dtype=dtype, with_grouped=False)
                     units.append(gs)
-    # Two measured alternatives of the fp16 kernel, kept behind a tuning entry point so that the comparison can be
-    # repeated: 32 x 32 accumulator blocks (v_mfma_f32_32x32x16) with four waves of 128 x 128, and with eight waves of
+    # The 256 x 256 tile on 32 x 32 accumulator blocks (v_mfma_f32_32x32x16), four waves of 128 x 128: behind at the
+    # socket's power limit (8192^3: 1.29 against 1.36 PFLOP/s) and ahead away from it, so launches of one round that
+    # leaves a third of the CUs idle take it (kSparseRoundBelow in lego_hip_abi.hip); the fp16 build for operands as
+    # given is also behind the tuning entry point, beside a second alternative kept for the comparison: eight waves of
     # 128 x 64 per workgroup, two per SIMD with 128 accumulator registers each (a second wave to issue from while one
-    # waits).  8192^3: 1.29 and 1.28 PFLOP/s against 1.36.
-    g32, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK["f16"]), dtype="f16", with_grouped=False, suffix="_m32")
+    # waits; 8192^3 1.28).
+    g32 = [gemm.emit(**dict(GEMM, bk=GEMM_BK[dtype]), trans_a=ta, trans_b=tb, dtype=dtype, with_grouped=False, suffix="_m32")[0]
+           for dtype in GEMM_SPARSE_ROUND_DTYPES for ta in (False, True) for tb in (False, True)]
     g8, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK["f16"], waves=GEMM_WAVES_TWO_PER_SIMD), dtype="f16", with_grouped=False)
     # A measurement build of the fp16 kernels as launched (same tiles, same schedules): lane 0 of every workgroup
     # records the real-time counter at seven points of its tile and the CU it ran on, for the per-phase tables of
     # bench.py --only timeline.
     gst, _ = gemm.emit(**dict(GEMM, bk=GEMM_BK["f16"]), dtype="f16", block=GEMM_MFMA_BLOCK["f16"], with_grouped=True,
                        with_split=True, suffix="_stamps", stamps=True)
-    units += [g32, g8, gst]
+    units += g32 + [g8, gst]
     units.append(gemm.emit_any())
     lbs, mlb = layernorm_bwd.emit()
     units += lbs
@@ -273,7 +277,8 @@ def collect():
           f"hipError_t lego_grouped_gemm_f16_t{GEMM_SMALL_TILE}x{GEMM_SMALL_TILE}_launch(const void* const*, "
           "const void* const*, void* const*, const int*, int, hipStream_t);",
           "hipError_t lego_gemm_f16_nn_w2x4_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);",
-          "hipError_t lego_gemm_f16_nn_m32_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);",
+          *[f"hipError_t lego_gemm_{d}_{v}_m32_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);"
+            for d in GEMM_SPARSE_ROUND_DTYPES for v in ("nn", "nt", "tn", "tt")],
           "hipError_t lego_gemm_f16_nn_stamps_launch(const void*, const void*, void*, int, int, int, int, hipStream_t);",
           "hipError_t lego_grouped_gemm_f16_stamps_launch(const void* const*, const void* const*, void* const*, "
           "const int*, int, hipStream_t);",

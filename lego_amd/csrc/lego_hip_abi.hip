@@ -599,7 +599,7 @@ typedef hipError_t (*gemm_launcher)(const void*, const void*, void*, int, int, i
 struct GemmKernels {
   gemm_launcher big[4];     // 256 x 256 tiles, one workgroup per CU; index 2*trans_a + trans_b
   gemm_launcher small[4];   // 128 x 128 tiles, two workgroups per CU (null: not built for this type)
-  gemm_launcher sparse[4];  // 256 x 256 tiles on 32x32x16 MFMAs, for launches that leave many CUs idle (null: not built)
+  gemm_launcher sparse[4];  // 256 x 256 tiles on 32x32x16 MFMAs, for launches that leave many CUs idle (null: not built for this type)
 };
 // Fewer 256 x 256 tiles than this and the 128 x 128 kernel, with four times as many workgroups,
 // keeps more of the 256 CUs busy than its higher LDS traffic per flop costs.
@@ -684,17 +684,15 @@ typedef hipError_t (*splitk_launcher)(const void*, const void*, void*, int, int,
   {{lego_gemm_##DT##_nn_launch, lego_gemm_##DT##_nt_launch, lego_gemm_##DT##_tn_launch,              \
     lego_gemm_##DT##_tt_launch},                                                                       \
    {lego_gemm_##DT##_nn_t128x128_launch, lego_gemm_##DT##_nt_t128x128_launch,                         \
-    lego_gemm_##DT##_tn_t128x128_launch, lego_gemm_##DT##_tt_t128x128_launch}}
+    lego_gemm_##DT##_tn_t128x128_launch, lego_gemm_##DT##_tt_t128x128_launch},                         \
+   {lego_gemm_##DT##_nn_m32_launch, lego_gemm_##DT##_nt_m32_launch, lego_gemm_##DT##_tn_m32_launch,  \
+    lego_gemm_##DT##_tt_m32_launch}}
 }  // namespace
 
 int lego_hip_gemm_f16_ex(const void* a, const void* b, void* c, int M, int N, int K, int trans_a, int trans_b,
                          int activation, void* stream)
 {
-  static const GemmKernels k = [] {
-    GemmKernels t = LEGO_GEMM_KERNELS(f16);
-    t.sparse[0] = lego_gemm_f16_nn_m32_launch;      // built for operands as given only
-    return t;
-  }();
+  static const GemmKernels k = LEGO_GEMM_KERNELS(f16);
   return gemm_ex(k, 0, a, b, c, M, N, K, trans_a, trans_b, activation, stream);
 }
 

@@ -595,6 +595,26 @@ def test_gemm_launches_that_leave_cus_idle(ops, M, N, K):
     assert torch.equal(act, torch.where(want >= 0, want, 0.01 * want).half())
 
 
+@pytest.mark.parametrize("kind", ["f16", "bf16", "bf16_to_f16"])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("M,N,K", [(2304, 4096, 64), (2296, 4088, 72)])
+def test_gemm_sparse_round_in_every_layout_and_type(ops, kind, ta, tb, M, N, K):
+    """144 tiles of 256 x 256, whole and ragged: the 32x32x16 builds of all four operand layouts and the three 16-bit
+    type combinations, with the fused activation.  Operands of -1, 0, 1: every sum is exact in bfloat16 too."""
+    print(f"gemm sparse round {kind} ta={ta} tb={tb} {M}x{N}x{K}", flush=True)
+    dtype = torch.float16 if kind == "f16" else torch.bfloat16
+    out = torch.bfloat16 if kind == "bf16" else torch.float16
+    g = _gen(73)
+    a = torch.randint(-1, 2, (M, K), generator=g).to(dtype)
+    b = torch.randint(-1, 2, (K, N), generator=g).to(dtype)
+    want = a.float() @ b.float()
+    ad = a.t().contiguous().cuda().t() if ta else a.cuda()
+    bd = b.t().contiguous().cuda().t() if tb else b.cuda()
+    assert torch.equal(ops.matmul(ad, bd, out_dtype=out).cpu().float(), want)
+    act = ops.matmul(ad, bd, activation="leaky_relu", out_dtype=out).cpu()
+    assert torch.equal(act, torch.where(want >= 0, want, 0.01 * want).to(out))
+
+
 def test_grouped_gemm_matches_oracle(ops):
     print("grouped gemm", flush=True)
     g = _gen(5)
