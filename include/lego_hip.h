@@ -243,7 +243,8 @@ int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const 
 /* Tuning entry point: C = A * B (fp16, row-major, N and K multiples of 8, 16-byte aligned bases) on 256 x 256 tiles
  * with the kernel chosen by the caller: variant 0 = what lego_hip_gemm_f16 launches for large products (four waves of
  * 128 x 128, one per SIMD with 256 accumulator registers, v_mfma_f32_16x16x32_f16), 1 = the same workgroup with
- * v_mfma_f32_32x32x16_f16, 2 = eight waves of 128 x 64, two per SIMD with 128 accumulator registers each
+ * v_mfma_f32_32x32x16_f16 (what it launches for 129 to 175 tiles, one round of workgroups that leaves a third of the
+ * CUs idle), 2 = eight waves of 128 x 64, two per SIMD with 128 accumulator registers each
  * (v_mfma_f32_32x32x16_f16), 3 = the measurement build of variant 0 (below).  Used by the benchmark to compare
  * them.  No counterpart in the reference. */
 int lego_hip_gemm_f16_variant(const void* a, const void* b, void* c, int M, int N, int K, int variant, void* stream);
