@@ -492,10 +492,14 @@ def main():
             ms_probe8 = timed(lambda: runtime.call("lego_hip_mfma_probe", p(ops8), p(probe_sink), 5, probe_iters // 2, probe_wgs, stream),
                               steps=max(5, K // 5), warmup=max(2, W // 5))
             ceiling8 = probe_wgs * (probe_iters // 2) * 8388608.0 / ms_probe8 / 1e9
+            ms_probe8s = timed(lambda: runtime.call("lego_hip_mfma_probe", p(ops8), p(probe_sink), 7, probe_iters // 4, probe_wgs, stream),
+                               steps=max(5, K // 5), warmup=max(2, W // 5))
             kernels["mfma_ceiling_fp8_e5m2"] = dict(
                 ms=ms_probe8, tflops=ceiling8, frac_mfma=ceiling8 / MFMA_FP8_PEAK_TFLOPS,
-                note="v_mfma_f32_32x32x64_f8f6f4 only, operands randn cast to e5m2 held in registers, 256 workgroups of "
-                     "four waves: what the part sustains with the pipe full")
+                tflops_16x16x128=probe_wgs * (probe_iters // 4) * 16777216.0 / ms_probe8s / 1e9,
+                note="v_mfma_f32_32x32x64_f8f6f4 only (the 8-bit GEMM kernels' instruction), operands randn cast to e5m2 "
+                     "held in registers, 256 workgroups of four waves: what the part sustains with the pipe full; "
+                     "tflops_16x16x128 = the same with v_mfma_f32_16x16x128_f8f6f4")
             kernels["next_gemm_fp8_e5m2_8192"] = dict(ms=ms8, tflops=fl4 / ms8 / 1e9,
                                                       frac_mfma=fl4 / ms8 / 1e9 / MFMA_FP8_PEAK_TFLOPS,
                                                       achievable_tflops=ceiling8, frac_of_achievable=fl4 / ms8 / 1e9 / ceiling8,

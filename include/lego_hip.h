@@ -298,6 +298,8 @@ int lego_hip_hbm_probe(const void* in, void* out, unsigned long long bytes, int 
  *   accumulator registers each, a 128 x 64 block per wave: 4194304 / 2097152 flop per round and workgroup).
  *   shape 5 / 6: v_mfma_f32_32x32x64_f8f6f4 with the operands' bytes read as OCP e5m2 / e4m3 (16 per round and
  *   wave over 4 x 4 blocks: 8388608 flop per round and workgroup; the same workgroups * 64 KiB of operands).
+ *   shape 7: v_mfma_f32_16x16x128_f8f6f4 on the operands of shape 5 (e5m2; 64 per round and wave over 8 x 8 blocks:
+ *   16777216 flop per round and workgroup).
  * sink: workgroups * 512 floats (a sum per lane, so that the work is not optimised away).  bench.py runs it with
  * operands of the GEMM benchmark's distribution and reports the rate as what the socket's power limit leaves to
  * an fp16 GEMM whose data movement costs nothing. */

@@ -229,6 +229,41 @@ __global__ void __launch_bounds__(256) lego_mfma_probe_8bit_kernel(const probe_i
   sink[static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x] = total;
 }
 
+// The same operands through v_mfma_f32_16x16x128_f8f6f4 on 8 x 8 blocks (shape 7): the fragments of the second four
+// block rows and columns are those of the first four with their halves swapped, in registers of their own
+__global__ void __launch_bounds__(256) lego_mfma_probe_8bit_16x16_kernel(const probe_int8* __restrict__ operands, float* __restrict__ sink, unsigned iters)
+{
+  const probe_int8* mine = operands + (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 8;
+  probe_int8 fa[8], fb[8];
+#pragma unroll
+  for (int f = 0; f < 4; ++f) {
+    fa[f] = mine[f];
+    fb[f] = mine[4 + f];
+    fa[4 + f] = __builtin_shufflevector(fa[f], fa[f], 4, 5, 6, 7, 0, 1, 2, 3);
+    fb[4 + f] = __builtin_shufflevector(fb[f], fb[f], 4, 5, 6, 7, 0, 1, 2, 3);
+  }
+  probe_float4 acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = probe_float4{0.0f, 0.0f, 0.0f, 0.0f};
+  for (unsigned it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], fa[i], acc[i][j], 1, 1, 0, 0, 0, 0);
+  }
+  float total = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) total += acc[i][j][r];
+  sink[static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x] = total;
+}
+
 typedef unsigned u32x4w __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4w_any __attribute__((ext_vector_type(4), aligned(2)));     // the same 16 bytes at any 2-byte element
 
@@ -1163,12 +1198,13 @@ int lego_hip_hbm_probe(const void* in, void* out, unsigned long long bytes, int 
 
 int lego_hip_mfma_probe(const void* operands, float* sink, int shape, int iters, int workgroups, void* stream)
 {
-  if (!usable(operands) || !usable(sink) || shape < 0 || shape > 6 || iters <= 0 || workgroups <= 0) return kInvalid;
+  if (!usable(operands) || !usable(sink) || shape < 0 || shape > 7 || iters <= 0 || workgroups <= 0) return kInvalid;
   const dim3 grid(static_cast<unsigned>(workgroups)), block(256);
   const probe_half8* src = static_cast<const probe_half8*>(operands);
   hipStream_t s = as_stream(stream);
   if (shape == 5) hipLaunchKernelGGL(lego_mfma_probe_8bit_kernel<1>, grid, block, 0, s, static_cast<const probe_int8*>(operands), sink, static_cast<unsigned>(iters));
   else if (shape == 6) hipLaunchKernelGGL(lego_mfma_probe_8bit_kernel<0>, grid, block, 0, s, static_cast<const probe_int8*>(operands), sink, static_cast<unsigned>(iters));
+  else if (shape == 7) hipLaunchKernelGGL(lego_mfma_probe_8bit_16x16_kernel, grid, block, 0, s, static_cast<const probe_int8*>(operands), sink, static_cast<unsigned>(iters));
   else if (shape == 3) hipLaunchKernelGGL(lego_mfma_probe2_kernel<3>, grid, dim3(512), 0, s, src, sink, static_cast<unsigned>(iters));
   else if (shape == 4) hipLaunchKernelGGL(lego_mfma_probe2_kernel<4>, grid, dim3(512), 0, s, src, sink, static_cast<unsigned>(iters));
   else if (shape == 0) hipLaunchKernelGGL(lego_mfma_probe_kernel<0>, grid, block, 0, s, src, sink, static_cast<unsigned>(iters));
