@@ -240,6 +240,13 @@ int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const 
                                    float* mean, float* rstd, int M, int N, float eps,
                                    int waves_per_row, void* stream);
 
+/* What lego_hip_gemm_f16_ex and lego_hip_gemm_bf16*_ex launch for a product whose operands lie in whole 16-byte chunks,
+ * without touching a device: plan2[0] = side of the workgroup's tile (256 or 128), plan2[1] = side of the MFMA's
+ * accumulator block (16: v_mfma_f32_16x16x32, 32: v_mfma_f32_32x32x16).  No counterpart in the reference (its
+ * autotuner picks among tile configurations at run time, matmul_sympy.py:98-165); it is there so that the choice can be
+ * checked on the host. */
+int lego_hip_gemm_plan(int M, int N, int K, int* plan2);
+
 /* Tuning entry point: C = A * B (fp16, row-major, N and K multiples of 8, 16-byte aligned bases) on 256 x 256 tiles
  * with the kernel chosen by the caller: variant 0 = what lego_hip_gemm_f16 launches for large products (four waves of
  * 128 x 128, one per SIMD with 256 accumulator registers, v_mfma_f32_16x16x32_f16), 1 = the same workgroup with

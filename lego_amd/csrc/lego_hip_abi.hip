@@ -668,6 +668,15 @@ inline bool small_tiles_fill_better(int M, int N, long tiles)
   return small_time < big_time;
 }
 
+// Which build a product in whole 16-byte chunks takes: 0 = 256 x 256 tiles on the type's own MFMA, 1 = 128 x 128 tiles,
+// 2 = 256 x 256 tiles on the 32x32x16 MFMA (16-bit operands: one round that leaves a third of the CUs idle).
+inline int gemm_choice(int M, int N, bool has_small, bool has_sparse)
+{
+  const long tiles = static_cast<long>((M + LEGO_GEMM_BM - 1) / LEGO_GEMM_BM) * ((N + LEGO_GEMM_BN - 1) / LEGO_GEMM_BN);
+  if (has_small && small_tiles_fill_better(M, N, tiles)) return 1;
+  return has_sparse && tiles < kSparseRoundBelow ? 2 : 0;
+}
+
 int gemm_ex(const GemmKernels& k, int element, const void* a, const void* b, void* c, int M, int N, int K,
             int trans_a, int trans_b, int activation, void* stream, int bk = LEGO_GEMM_BK, int chunk = 8)
 {
@@ -688,10 +697,9 @@ int gemm_ex(const GemmKernels& k, int element, const void* a, const void* b, voi
     return ok_or(lego_gemm_any_launch(a, b, c, M, N, K, trans_a ? 1 : 0, trans_b ? 1 : 0, activation, element,
                                       as_stream(stream)));
   }
-  const long tiles = static_cast<long>((M + LEGO_GEMM_BM - 1) / LEGO_GEMM_BM) * ((N + LEGO_GEMM_BN - 1) / LEGO_GEMM_BN);
   const int layout = (trans_a ? 2 : 0) + (trans_b ? 1 : 0);
-  const gemm_launcher* by_layout = small_tiles_fill_better(M, N, tiles) && k.small[layout] != nullptr ? k.small
-                                   : tiles < kSparseRoundBelow && k.sparse[layout] != nullptr ? k.sparse : k.big;
+  const int choice = gemm_choice(M, N, k.small[layout] != nullptr, k.sparse[layout] != nullptr);
+  const gemm_launcher* by_layout = choice == 1 ? k.small : choice == 2 ? k.sparse : k.big;
   return ok_or(by_layout[layout](a, b, c, M, N, K, activation, as_stream(stream)));
 }
 
@@ -1117,6 +1125,15 @@ int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* 
   if (plan.kind == 1) return ok_or(lego_grouped_gemm_f16_t128x128_launch(a, b, c, sizes3, groups, as_stream(stream)));
   if (plan.split == 0) return ok_or(lego_grouped_gemm_f16_launch(a, b, c, sizes3, groups, as_stream(stream)));
   return ok_or(lego_grouped_gemm_f16_split_launch(a, b, c, sizes3, groups, plan.split, as_stream(stream)));
+}
+
+int lego_hip_gemm_plan(int M, int N, int K, int* plan2)
+{
+  if (plan2 == nullptr || M <= 0 || N <= 0 || K <= 0) return kInvalid;
+  const int choice = gemm_choice(M, N, true, true);
+  plan2[0] = choice == 1 ? 128 : 256;
+  plan2[1] = choice == 0 ? 16 : 32;
+  return 0;
 }
 
 int lego_hip_grouped_gemm_f16_plan(const int* sizes3, int groups, int* plan3)

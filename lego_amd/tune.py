@@ -113,7 +113,9 @@ def tune_gemm(torch, lib, ns):
         a = (torch.randn(M, K, device="cuda") / math.sqrt(K)).half()
         b = (torch.randn(K, N, device="cuda") / math.sqrt(K)).half()
         c = torch.empty(M, N, device="cuda", dtype=torch.half)
-        out = []
+        plan = (ctypes.c_int * 2)()
+        assert lib.lego_hip_gemm_plan(M, N, K, plan) == 0
+        out = [f"plan: {plan[0]} x {plan[0]} tiles, {plan[1]} x {plan[1]} MFMA blocks"]
         for v, label in names.items():
             def fn():
                 return lib.lego_hip_gemm_f16(p(a), p(b), p(c), M, N, K, stream) if v < 0 else \

@@ -97,3 +97,28 @@ def test_plan_keeps_whole_rounds_whole_and_small_sets_on_small_tiles():
     assert _plan([(1024, 512, 256), (512, 512, 512)])[0] == 128    # a handful of tiles: 128 x 128 tiles
     with pytest.raises(runtime.LegoHipError):
         _plan([(0, 256, 64)])
+
+
+def _gemm_plan(M, N, K=4096):
+    out = (ctypes.c_int * 2)()
+    runtime.call("lego_hip_gemm_plan", M, N, K, out)
+    return tuple(out)
+
+
+def test_gemm_plan_follows_the_measured_crossovers():
+    """The single-product dispatch, on the host: (tile side, MFMA block side) for the shapes its thresholds were
+    measured on."""
+    big, small, sparse = (256, 16), (128, 32), (256, 32)
+    assert _gemm_plan(8192, 8192) == big and _gemm_plan(4096, 4096) == big          # whole rounds
+    assert _gemm_plan(2048, 2048) == small and _gemm_plan(2048, 4096) == small        # up to 128 big tiles
+    # one round that leaves a third of the CUs idle: the 32x32x16 build up to 175 tiles
+    assert _gemm_plan(3072, 3072) == sparse and _gemm_plan(2304, 4096) == sparse and _gemm_plan(2560, 4096) == sparse
+    assert _gemm_plan(2816, 4096) == big and _gemm_plan(3584, 3584) == big
+    # a mostly empty second round: small tiles while they make the estimate in rounds shorter
+    assert _gemm_plan(4352, 4096) == small and _gemm_plan(5120, 4096) == small and _gemm_plan(4608, 4608) == small
+    assert _gemm_plan(6144, 4096) == big and _gemm_plan(5120, 5120) == big and _gemm_plan(6144, 6144) == big
+    assert _gemm_plan(7168, 4096) == big
+    # ragged tiles count as whole ones
+    assert _gemm_plan(3071, 3065) == sparse and _gemm_plan(8184, 8184) == big
+    with pytest.raises(runtime.LegoHipError):
+        _gemm_plan(0, 256)
