@@ -247,6 +247,12 @@ int lego_hip_layernorm_fwd_f16_wpr(const void* x, void* y, const void* w, const 
  * checked on the host. */
 int lego_hip_gemm_plan(int M, int N, int K, int* plan2);
 
+/* The team that lego_hip_softmax_f16 and lego_hip_layernorm_fwd_f16 give a row of a matrix of M rows of N fp16
+ * elements in whole 16-byte vectors on 16-byte aligned bases (N a multiple of 8, at most 32768): waves per row, the
+ * argument that the _wpr entry points above take.  Host only; no counterpart in the reference (its softmax sizes one
+ * program from BLOCK_SIZE with a fixed num_warps = 8, softmax.py:97-122). */
+int lego_hip_rows_f16_plan(int M, int N, int* waves_per_row);
+
 /* Tuning entry point: C = A * B (fp16, row-major, N and K multiples of 8, 16-byte aligned bases) on 256 x 256 tiles
  * with the kernel chosen by the caller: variant 0 = what lego_hip_gemm_f16 launches for large products (four waves of
  * 128 x 128, one per SIMD with 256 accumulator registers, v_mfma_f32_16x16x32_f16), 1 = the same workgroup with

@@ -1127,6 +1127,13 @@ int lego_hip_grouped_gemm_f16(const void* const* a, const void* const* b, void* 
   return ok_or(lego_grouped_gemm_f16_split_launch(a, b, c, sizes3, groups, plan.split, as_stream(stream)));
 }
 
+int lego_hip_rows_f16_plan(int M, int N, int* waves_per_row)
+{
+  if (waves_per_row == nullptr || M <= 0 || N <= 0 || N % 8 != 0 || N > LEGO_ROWWISE_MAX_N) return kInvalid;
+  *waves_per_row = lego_rowwise_f16_wpr(M, N);
+  return 0;
+}
+
 int lego_hip_gemm_plan(int M, int N, int K, int* plan2)
 {
   if (plan2 == nullptr || M <= 0 || N <= 0 || K <= 0) return kInvalid;

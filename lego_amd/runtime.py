@@ -34,6 +34,7 @@ SIGNATURES = {
     "lego_hip_gemm_f16": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "lego_hip_gemm_f16_variant": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "lego_hip_gemm_plan": [_c_int, _c_int, _c_int, ctypes.POINTER(_c_int)],
+    "lego_hip_rows_f16_plan": [_c_int, _c_int, ctypes.POINTER(_c_int)],
     "lego_hip_gemm_f16_act": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "lego_hip_gemm_f16_ex": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                              _c_void_p],

@@ -122,3 +122,23 @@ def test_gemm_plan_follows_the_measured_crossovers():
     assert _gemm_plan(3071, 3065) == sparse and _gemm_plan(8184, 8184) == big
     with pytest.raises(runtime.LegoHipError):
         _gemm_plan(0, 256)
+
+
+def _rows_plan(M, N):
+    out = ctypes.c_int()
+    runtime.call("lego_hip_rows_f16_plan", M, N, ctypes.byref(out))
+    return out.value
+
+
+def test_row_team_sizes_follow_the_measured_crossovers():
+    """Waves per row of the fp16 softmax and LayerNorm forward, on the host, for the shapes the thresholds were
+    measured on."""
+    assert _rows_plan(8192, 8192) == 8 and _rows_plan(8192, 16384) == 8 and _rows_plan(8192, 6152) == 8    # long rows, tall
+    assert _rows_plan(2048, 8192) == 4 and _rows_plan(8192, 6144) == 4 and _rows_plan(8192, 4096) == 4
+    assert _rows_plan(4096, 4096) == 2 and _rows_plan(2500, 3080) == 2        # one round of workgroups instead of two
+    assert _rows_plan(8192, 2048) == 1 and _rows_plan(65536, 1024) == 1 and _rows_plan(32768, 1536) == 1
+    assert _rows_plan(16384, 2048) == 2 and _rows_plan(65536, 1600) == 2      # four vectors per lane of one wave, very tall
+    assert _rows_plan(512, 32768) == 16 and _rows_plan(600, 20488) == 16
+    for bad in ((8192, 8191), (0, 8), (8, 32776)):
+        with pytest.raises(runtime.LegoHipError):
+            _rows_plan(*bad)
